@@ -1,0 +1,154 @@
+"""Benchmark of the TTT operation on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1|c2|c4] [--no-cpu-baseline]
+
+One step = forward + backward of block_causal_lact_swiglu over one batch of seeded synthetic input
+that is resident in HBM before the timed region.  Prints one JSON line (metric: tokens/s, tokens = B*L).
+"""
+import argparse
+import ctypes
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA peak
+PEAK_HBM_GBS = 8000.0
+
+CONFIGS = {
+    # name: (B, H, L, d, dh, chunk, seed, text)
+    "c1": (4, 4, 4096, 384, 384, 2048, 1001,
+           "config 1: block_causal_lact_swiglu fwd+bwd, 760M shape B=4 H=4 (b=16), L=4096, d=dh=384, chunk 2048, "
+           "Muon NS5 + momentum 0.9, bf16 activations / fp32 fast weights"),
+    "c2": (1, 4, 32768, 384, 384, 2048, 1002,
+           "config 2: block_causal_lact_swiglu fwd+bwd, B=1 H=4 (b=4), L=32768, d=dh=384, chunk 2048, Muon + momentum"),
+    "c4": (1, 12, 32760, 128, 256, 4680, 1004,
+           "config 4: block_causal_lact_swiglu fwd+bwd, video shape b=12, L=32760, d=128, dh=256, chunk 4680, Muon + momentum"),
+}
+
+
+def algorithmic_flops(b, L, d, dh, C, ns_steps=5):
+    """Counted FLOPs of fwd+bwd (multiply-add = 2; backward = 2x forward; recompute, momentum, renorm and
+    pointwise work not counted): F_apply = 6 d dh T, F_update = 12 d dh T, F_ns = 3 steps (4 r^2 c + 2 r^3)."""
+    n_chunks = max(1, math.ceil(L / C))
+    n_upd = n_chunks - 1
+    r, c = min(d, dh), max(d, dh)
+    f_apply = 6.0 * d * dh * L
+    f_update = 12.0 * d * dh * (n_upd * C)
+    f_ns = 3.0 * ns_steps * (4.0 * r * r * c + 2.0 * r ** 3) * n_upd
+    return 3.0 * b * (f_apply + f_update + f_ns)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", default="c1", choices=sorted(CONFIGS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernel-profile", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures the one-GPU operation only: heads (b = B*H) are independent, so N GPUs would each run "
+              "a slice of b with no communication; run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import lact_amd
+    from lact_amd import _lib
+    from oracle import lact_oracle as O
+
+    B, H, L, d, dh, C, seed, text = CONFIGS[args.config]
+    b = B * H
+    inp = O.make_inputs(b, L, d, dh, seed=seed, act_dtype=torch.bfloat16, distinct_heads=H, momentum_value=0.9)
+    order = ("w0", "w1", "w2", "q", "k", "v", "lr0", "lr1", "lr2")
+    names = list(order) + ["momentum"]
+    dev = {n: inp[n].to("cuda:0").requires_grad_(True) for n in names}
+    go = torch.randn(b, L, d, generator=torch.Generator().manual_seed(seed + 1)).bfloat16().to("cuda:0")
+
+    def step():
+        for t in dev.values():
+            t.grad = None
+        out = lact_amd.block_causal_lact_swiglu(*[dev[n] for n in order], C, True, dev["momentum"])
+        out.backward(go)
+        return out
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    tokens_per_s = B * L * args.steps / dt
+    flops = algorithmic_flops(b, L, d, dh, C)
+    op_tflops = flops / (ms_per_step * 1e-3) / 1e12
+
+    res = {
+        "metric": "TTT-layer tokens/sec fwd+bwd at 760M shape, 1 GPU; MFMA util % of bf16 peak",
+        "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic (seeded N(0,1) q,k,v; L2-normalised q,k; random-init fast weights)",
+        "config": {"workload": text, "tokens_per_step": B * L, "algorithmic_gflop_per_step": flops / 1e9},
+        "op_tflops": op_tflops, "op_frac_of_bf16_peak": op_tflops / PEAK_BF16_TFLOPS,
+    }
+
+    # ---- per-kernel durations: the same K steps again with HIP events around every launch, on the stream
+    #      the kernels run on (a second pass, so that the events do not perturb `value`)
+    if not args.no_kernel_profile:
+        Lb = _lib.lib()
+        Lb.lact_profile_enable(1)
+        for _ in range(args.steps):
+            step()
+        buf = ctypes.create_string_buffer(1 << 20)
+        _lib.check(Lb.lact_profile_report(buf, len(buf)))
+        Lb.lact_profile_enable(0)
+        rows = json.loads(buf.value.decode())
+        by_kernel = {}
+        for r in rows:
+            k = by_kernel.setdefault(r["kernel"], {"launches": 0, "ms": 0.0, "flops": 0.0})
+            k["launches"] += r["launches"]; k["ms"] += r["ms"]; k["flops"] += r["flops"]
+        total_ms = sum(k["ms"] for k in by_kernel.values())
+        dom_name, dom = max(((n, k) for n, k in by_kernel.items() if k["flops"] > 0), key=lambda x: x[1]["ms"])
+        avg_ms = dom["ms"] / dom["launches"]
+        achieved = dom["flops"] / dom["launches"] / (avg_ms * 1e-3) / 1e12
+        res["roofline"] = {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                           "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None, "kernel": dom_name,
+                           "avg_launch_ms": avg_ms, "launches_per_step": dom["launches"] / args.steps,
+                           "share_of_kernel_time": dom["ms"] / total_ms}
+        res["kernels"] = sorted(
+            [{"kernel": r["kernel"], "site": r["site"], "launches_per_step": r["launches"] / args.steps,
+              "ms_per_step": r["ms"] / args.steps,
+              "tflops": (r["flops"] / (r["ms"] * 1e-3) / 1e12) if r["ms"] > 0 and r["flops"] > 0 else None}
+             for r in rows], key=lambda r: -r["ms_per_step"])
+        res["kernel_ms_per_step"] = total_ms / args.steps
+
+    # ---- CPU baseline: the oracle (a restatement of the reference's non-fused PyTorch op) on the host cores
+    if not args.no_cpu_baseline:
+        cb = b if args.config == "c1" else min(b, 4)   # bounded sample: the first `cb` heads, forward + backward
+        cpu = {n: inp[n][:cb].clone().requires_grad_(True) for n in names}
+        gc = go[:cb].cpu()
+        t0 = time.perf_counter()
+        reps = 0
+        while reps < 1 or (time.perf_counter() - t0 < 12.0 and reps < 40):
+            for t in cpu.values():
+                t.grad = None
+            o = O.block_causal_lact_swiglu(*[cpu[n] for n in order], C, True, cpu["momentum"], num=O.Numerics(autocast=True))
+            o.backward(gc)
+            reps += 1
+        ct = (time.perf_counter() - t0) / reps
+        res["cpu_baseline"] = {"value": (B * L) * (cb / b) / ct, "unit": "tokens/s", "cores": torch.get_num_threads(),
+                               "kind": "port",
+                               "sample": f"first {cb} of {b} heads of the same workload, fwd+bwd, {reps} run(s), "
+                                         f"{ct:.2f} s each; tokens scaled by {cb}/{b}; host has {os.cpu_count()} logical CPUs"}
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,116 @@
+/* C ABI of the MI355X large-chunk TTT library (liblact_hip.so).
+ *
+ * The reference has no FFI: its boundary for this path is a set of Python functions of tensors
+ * called from the layers' forward().  Every entry point below is what a binding of that boundary
+ * needs; none takes a torch type.  All pointers except `steps` and `ns_coeffs` are device
+ * pointers; sizes are element counts unless a name says bytes; all calls enqueue work on `stream`
+ * (a hipStream_t passed as void*) and return without synchronising.  Return value 0 = success,
+ * negative = error; lact_last_error() gives the message of the calling thread's last failure.
+ *
+ * Layout (reference LLM layout, lact_llm/lact_model/ttt_operation.py:71-105):
+ *   w0, w2: [b, dh, d]   w1: [b, d, dh]   fp32, contiguous
+ *   q: [b, q_len, d]  k, v: [b, kv_len, d]   bf16 or fp32 (act_dtype), last dim contiguous,
+ *      row stride *_ld and batch stride *_bs given in elements
+ *   lr0, lr1, lr2, momentum: [b, kv_len] fp32 contiguous
+ *   out: [b, out_len, d] act_dtype
+ * d and dh must be multiples of 8; key and value dims are equal (every configuration of the
+ * reference has dk == dv).
+ */
+#ifndef LACT_HIP_H
+#define LACT_HIP_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { LACT_BF16 = 0, LACT_F32 = 1 };
+enum { LACT_UPDATE = 0, LACT_APPLY = 1 };
+/* Newton-Schulz numerics.  AUTOCAST: bf16 GEMM operands, fp32 accumulation and fp32 iterate, what
+ * ttt_operation.py:30-66 computes under torch.autocast(bf16).  PLAIN_BF16: the iterate itself is
+ * rounded to bf16 after every step, what the same code computes without autocast (:45 casts to bf16
+ * and nothing casts back).  FP32: no bf16 anywhere (fp32 MFMA); not a reference mode, used to check
+ * the closed-form backward against exact arithmetic. */
+enum { LACT_NS_AUTOCAST = 0, LACT_NS_PLAIN_BF16 = 1, LACT_NS_FP32 = 2 };
+
+/* One step of a test-time-training program.
+ * UPDATE: one fast-weight update from k, v, lr, momentum rows [start, end)
+ *         (ttt_operation.py:147-200; lact_nvs/lact_ttt.py:104-138).
+ * APPLY:  out rows [out_start, out_start + end - start) = f_w(q rows [start, end))
+ *         (ttt_operation.py:141-144; lact_nvs/lact_ttt.py:140-143).
+ * The reference's schedules are all sequences of these: block-causal = apply,update per chunk then
+ * a last apply (ttt_operation.py:124,202-212); bidirectional = update(all), apply(all)
+ * (bidirectional_lact_layer.py:118-158); NVS = the TTTOperator list (lact_ttt.py:10,101);
+ * AR video = apply, then update/apply pairs (ar_lact_swa_repeat.py:97-165). */
+typedef struct lact_step {
+  int32_t kind, start, end, out_start;
+} lact_step_t;
+
+typedef struct lact_desc {
+  int32_t b, d, dh;
+  int32_t q_len, kv_len, out_len;
+  int32_t act_dtype;
+  int32_t n_steps;
+  const lact_step_t* steps;      /* host memory */
+  int32_t ns_steps;              /* Newton-Schulz iterations; -1 = Muon off; 0 = cast + normalise only */
+  const float* ns_coeffs;        /* host memory, 3*ns_steps floats (a,b,c per iteration;
+                                    ttt_operation.py:51-57 or lact_ttt.py:51) */
+  int32_t use_momentum;          /* ttt_operation.py:170-179 */
+  int32_t prenorm;               /* ttt_operation.py:219-364 (un-normalised accumulator) */
+  int32_t weight_norm;           /* ar_lact_swa_repeat.py:149-153 */
+  int32_t detach_norms;          /* lact_ttt.py:96-98 */
+  int32_t muon_replaces_weight;  /* bidirectional_lact_layer.py:139-146: w_hat = NS(dw) + dw */
+  int32_t ns_mode;               /* LACT_NS_* */
+  int64_t q_bs, k_bs, v_bs, o_bs, do_bs;
+  int32_t q_ld, k_ld, v_ld, o_ld, do_ld;
+} lact_desc_t;
+
+const char* lact_last_error(void);
+int lact_version(void);
+
+/* Bytes of the two caller-owned buffers: `saved` lives from forward to backward (fast-weight
+ * versions, momentum states, Newton-Schulz iterates); `scratch` only during one call. */
+int lact_query_sizes(const lact_desc_t* desc, size_t* saved_bytes, size_t* scratch_bytes);
+
+/* Whole forward of one program.  Replaces block_causal_lact_swiglu / prenorm_block_causal_lact_swiglu
+ * (ttt_operation.py:71-214, 219-364), bidirectional_lact_swiglu (bidirectional_lact_layer.py:74-160),
+ * fast_weight_swish_glu_weight_norm_mini_batch_apply (lact_ttt.py:71-147) and the
+ * ar_fast_weight_swish_glu_weight_norm_mini_batch family (ar_lact_swa_repeat.py:23-296).
+ * w_out[3] / m_out[3] (each nullable, fp32, shapes of w0,w1,w2) receive the final fast weights and
+ * momentum states (lact_ttt.py:147; ar_lact_swa_repeat_sp.py:339). */
+int lact_forward(const lact_desc_t* desc, const float* w0, const float* w1, const float* w2, const void* q,
+                 const void* k, const void* v, const float* lr0, const float* lr1, const float* lr2,
+                 const float* momentum, void* out, float* const w_out[3], float* const m_out[3], void* saved,
+                 void* scratch, void* stream);
+
+/* Backward of the same program (the reference relies on autograd; closed forms as in
+ * lact_triton_kernels/lact_swiglu_ffn.py:46-76, lact_fw_grad.py:61-156, l2norm_triton_kernels.py:106-172).
+ * dout: gradient of `out` (act_dtype, strides do_ld/do_bs); dw_final[3]: gradient of the returned
+ * final weights (nullable).  Outputs: dw0,dw1,dw2 fp32; dq,dk,dv act_dtype contiguous [b,len,d];
+ * dlr0..2, dmomentum fp32 [b,kv_len].  dq, dk, dv, dlr*, dmomentum must be zero-filled by the caller
+ * (rows no step touches stay zero; rows used by several steps accumulate). */
+int lact_backward(const lact_desc_t* desc, const void* q, const void* k, const void* v, const float* lr0,
+                  const float* lr1, const float* lr2, const float* momentum, const void* dout,
+                  const float* const dw_final[3], const void* saved, void* scratch, float* dw0, float* dw1,
+                  float* dw2, void* dq, void* dk, void* dv, float* dlr0, float* dlr1, float* dlr2,
+                  float* dmomentum, void* stream);
+
+/* zeropower_via_newtonschulz5 (ttt_operation.py:30-66; with a repeated coefficient triple:
+ * lact_ttt.py:33-67, functions.py:38-72).  g, out: [n, rows, cols] fp32. */
+size_t lact_newton_schulz_workspace_bytes(int32_t n, int32_t rows, int32_t cols, int32_t steps);
+int lact_newton_schulz(int32_t n, int32_t rows, int32_t cols, const float* g, float* out, int32_t steps,
+                       const float* coeffs, int32_t ns_mode, void* workspace, void* stream);
+
+/* Per-launch timing with HIP events on the caller's stream (no counterpart in the reference, which
+ * times with wall-clock prints, lact_ar_video/minVid/train.py:458-460).  While enabled every kernel
+ * launch of lact_forward / lact_backward is bracketed by two events; lact_profile_report synchronises
+ * the device, writes a JSON array of {kernel, site, launches, ms, flops} into buf and resets the
+ * records.  Not thread-safe; meant for benchmarking. */
+int lact_profile_enable(int on);
+int lact_profile_report(char* buf, size_t cap);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

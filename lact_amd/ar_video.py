@@ -1,0 +1,68 @@
+"""Drop-ins for the operations of lact_ar_video/minVid/models/blocks/ar_lact_swa_repeat{,_sp}.py."""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import ops
+from ._lib import LACT_APPLY, LACT_UPDATE
+from .ops import NS_CLASSIC, Program, run_program
+
+
+def zeropower_via_newtonschulz5(G: torch.Tensor, steps: int) -> torch.Tensor:
+    """functions.py:38-72."""
+    return ops.newton_schulz(G, (NS_CLASSIC,) * steps, ns_mode=ops.NS_AUTOCAST if torch.is_autocast_enabled() else ops.NS_PLAIN_BF16)
+
+
+def _ar_steps(seq_len, q_len, mini_batch_size, update_length, update_every, num_repeat):
+    """ar_lact_swa_repeat.py:76-101,104-165."""
+    if update_length == -1:
+        update_length = seq_len
+    if mini_batch_size == -1:
+        mini_batch_size = update_length
+    if update_every == -1:
+        update_every = mini_batch_size * 2
+    first = update_every - mini_batch_size
+    steps = [(LACT_APPLY, 0, first, 0)]
+    for _ in range(num_repeat):
+        for s in range(first, update_length, update_every):
+            steps.append((LACT_UPDATE, s, s + mini_batch_size, 0))
+            steps.append((LACT_APPLY, s, min(s + update_every, q_len), s))
+    return tuple(steps)
+
+
+def ar_fast_weight_swish_glu_weight_norm_mini_batch_with_momentum(
+        w0, w1, w2, q, k, v, lr0, lr1, lr2, w_scale: float, num_repeat: int = 1, mini_batch_size: int = -1,
+        update_length: int = -1, update_every: int = -1, use_moun: bool = False, num_moun_iters: int = 3,
+        weight_norm: bool = True, fw_momentum: Optional[torch.Tensor] = None, use_momentum: bool = False):
+    """ar_lact_swa_repeat_sp.py:28-193.  Returns (output, w0, w1, w2)."""
+    prog = Program(steps=_ar_steps(k.shape[1], q.shape[1], mini_batch_size, update_length, update_every, num_repeat),
+                   out_len=q.shape[1], ns_coeffs=(NS_CLASSIC,) * num_moun_iters if use_moun else None,
+                   weight_norm=weight_norm, ns_mode=ops._ns_mode(q))
+    out, ws, _ = run_program(prog, w0, w1, w2, q, k, v, lr0 * w_scale, lr1 * w_scale, lr2 * w_scale,
+                             fw_momentum if use_momentum else None)
+    return (out,) + tuple(ws)
+
+
+def ar_fast_weight_swish_glu_weight_norm_mini_batch(
+        w0, w1, w2, q, k, v, lr0, lr1, lr2, w_scale: float, num_repeat: int = 1, mini_batch_size: int = -1,
+        update_length: int = -1, update_every: int = -1, use_moun: bool = False, num_moun_iters: int = 3,
+        weight_norm: bool = True):
+    """ar_lact_swa_repeat.py:23-168."""
+    return ar_fast_weight_swish_glu_weight_norm_mini_batch_with_momentum(
+        w0, w1, w2, q, k, v, lr0, lr1, lr2, w_scale, num_repeat, mini_batch_size, update_length, update_every,
+        use_moun, num_moun_iters, weight_norm)
+
+
+def ar_fast_weight_swish_glu_weight_norm_mini_batch_inference(
+        w0, w1, w2, q, k, v, lr0, lr1, lr2, w_scale: float, num_repeat: int = 1, mini_batch_size: int = -1,
+        do_update: bool = False, use_moun: bool = False, num_moun_iters: int = 3, weight_norm: bool = True):
+    """ar_lact_swa_repeat.py:172-296: optional repeated update on the first mini-batch, then apply on all q."""
+    mb = k.shape[1] if mini_batch_size == -1 else mini_batch_size
+    steps = [(LACT_UPDATE, 0, mb, 0)] * (num_repeat if do_update else 0) + [(LACT_APPLY, 0, q.shape[1], 0)]
+    prog = Program(steps=tuple(steps), out_len=q.shape[1],
+                   ns_coeffs=(NS_CLASSIC,) * num_moun_iters if use_moun else None,
+                   weight_norm=weight_norm, ns_mode=ops._ns_mode(q))
+    out, ws, _ = run_program(prog, w0, w1, w2, q, k, v, lr0 * w_scale, lr1 * w_scale, lr2 * w_scale, None)
+    return (out,) + tuple(ws)

@@ -1,0 +1,852 @@
+// Host side of liblact_hip.so: validates a program, lays out the caller's buffers and enqueues the
+// kernels of the forward and backward passes on the caller's stream.  No allocation, no
+// synchronisation, no torch types.
+#include "../../include/lact_hip.h"
+
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "gemm_kernels.h"
+#include "state_kernels.h"
+
+using namespace lact;
+
+namespace {
+
+thread_local std::string g_err;
+int fail(const std::string& m) {
+  g_err = m;
+  return -1;
+}
+// ---- optional per-launch timing (HIP events on the caller's stream) ---------------------------------
+struct ProfRec {
+  const char* kernel;
+  const char* site;
+  double flops;
+  hipEvent_t e0, e1;
+};
+struct Profiler {
+  bool on = false;
+  std::vector<ProfRec> recs;
+  std::vector<hipEvent_t> pool;
+  hipEvent_t get() {
+    if (!pool.empty()) {
+      hipEvent_t e = pool.back();
+      pool.pop_back();
+      return e;
+    }
+    hipEvent_t e;
+    (void)hipEventCreate(&e);
+    return e;
+  }
+  void clear() {
+    for (auto& r : recs) {
+      pool.push_back(r.e0);
+      pool.push_back(r.e1);
+    }
+    recs.clear();
+  }
+};
+Profiler g_prof;
+struct ProfScope {
+  hipStream_t s;
+  hipEvent_t e1 = nullptr;
+  ProfScope(const char* kernel, const char* site, double flops, hipStream_t st) : s(st) {
+    if (!g_prof.on) return;
+    ProfRec r{kernel, site, flops, g_prof.get(), g_prof.get()};
+    (void)hipEventRecord(r.e0, s);
+    e1 = r.e1;
+    g_prof.recs.push_back(r);
+  }
+  ~ProfScope() {
+    if (e1) (void)hipEventRecord(e1, s);
+  }
+};
+// kern may contain template commas: pass it parenthesised
+#define LACT_LAUNCH(kname, site, flops, kern, grid, block, stream, ...)  \
+  do {                                                                  \
+    ProfScope ps_(kname, site, flops, stream);                          \
+    hipLaunchKernelGGL(kern, grid, block, 0, stream, __VA_ARGS__);      \
+  } while (0)
+
+template <typename T> const char* tname();
+template <> const char* tname<uint16_t>() { return "bf16"; }
+template <> const char* tname<float>() { return "f32"; }
+
+#define LACT_CHECK_LAUNCH()                                                     \
+  do {                                                                          \
+    hipError_t e_ = hipGetLastError();                                          \
+    if (e_ != hipSuccess) return fail(std::string("kernel launch failed: ") + hipGetErrorString(e_)); \
+  } while (0)
+
+using TSA = TileShape<128, 128, 2, 2>;  // two or three accumulators
+using TSB = TileShape<64, 128, 2, 2>;   // six accumulators (update backward)
+
+struct Bump {
+  size_t off = 0;
+  size_t take(size_t bytes) {
+    const size_t o = off;
+    off += (bytes + 255) & ~size_t(255);
+    return o;
+  }
+};
+
+int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+struct Split {
+  int n, len;
+};
+Split choose_split(int tokens, int tiles_total) {
+  int ns = std::max(1, ceil_div(512, std::max(1, tiles_total)));
+  ns = std::min(ns, std::max(1, tokens / 128));
+  int len = ceil_div(ceil_div(tokens, ns), 32) * 32;
+  return Split{ceil_div(tokens, len), len};
+}
+
+struct Plan {
+  lact_desc_t d;
+  std::vector<lact_step_t> steps;
+  std::vector<float> coeffs;
+  MatGeom g;
+  int nupd = 0, Tcap = 0, S = -1, esz = 2, nsz = 2, r = 0, c = 0, nblk = 1, lr_slots = 1, tiles = 1, nsplit_max = 1;
+  bool muon = false, bf16 = true, momentum = false;
+  size_t mat3 = 0;  // 3*b*elems
+  // saved
+  size_t s_n0, s_wf, s_wc, s_main, s_d, s_mbar, s_u, s_g16, s_norms, s_xb, s_ab, s_bb, saved_bytes;
+  // scratch
+  size_t t_h[6], t_partial, t_lrpart, t_xf[2], t_xbtmp, t_ss, t_dot, t_mdot, t_gwhat[2], t_gwcur, t_gmcarry, t_gc,
+      t_gxf[2], t_gxb[2], t_sg, t_gas, t_gn0, scratch_bytes;
+
+  int build(const lact_desc_t* desc) {
+    if (!desc) return fail("null descriptor");
+    d = *desc;
+    if (d.b <= 0 || d.d <= 0 || d.dh <= 0) return fail("b, d, dh must be positive");
+    if (d.d % 8 || d.dh % 8) return fail("d and dh must be multiples of 8");
+    if (d.act_dtype != LACT_BF16 && d.act_dtype != LACT_F32) return fail("act_dtype must be LACT_BF16 or LACT_F32");
+    bf16 = d.act_dtype == LACT_BF16;
+    esz = bf16 ? 2 : 4;
+    const int al = bf16 ? 8 : 4;
+    if (d.q_ld % al || d.k_ld % al || d.v_ld % al || d.o_ld % al || d.q_bs % al || d.k_bs % al || d.v_bs % al ||
+        d.o_bs % al)
+      return fail("row and batch strides must keep 16-byte alignment");
+    if (d.q_ld < d.d || d.k_ld < d.d || d.v_ld < d.d || d.o_ld < d.d) return fail("row stride smaller than d");
+    if (3LL * d.b > 65535) return fail("b too large (3*b must fit a grid dimension)");
+    if (d.n_steps <= 0 || !d.steps) return fail("empty program");
+    steps.assign(d.steps, d.steps + d.n_steps);
+    S = d.ns_steps;
+    muon = S >= 0;
+    if (S > 0 && !d.ns_coeffs) return fail("ns_coeffs missing");
+    if (S > 64) return fail("too many Newton-Schulz steps");
+    if (S > 0) coeffs.assign(d.ns_coeffs, d.ns_coeffs + 3 * S);
+    momentum = d.use_momentum != 0;
+    if (d.ns_mode < 0 || d.ns_mode > 2) return fail("ns_mode must be 0, 1 or 2");
+    nsz = d.ns_mode == LACT_NS_FP32 ? 4 : 2;
+    nupd = 0;
+    Tcap = 0;
+    for (const auto& s : steps) {
+      if (s.kind != LACT_UPDATE && s.kind != LACT_APPLY) return fail("step kind must be LACT_UPDATE or LACT_APPLY");
+      if (s.start < 0 || s.end <= s.start) return fail("empty or negative step range");
+      if (s.kind == LACT_UPDATE) {
+        if (s.end > d.kv_len) return fail("update range exceeds kv_len");
+        ++nupd;
+      } else {
+        if (s.end > d.q_len) return fail("apply range exceeds q_len");
+        if (s.out_start < 0 || s.out_start + (s.end - s.start) > d.out_len) return fail("apply output range exceeds out_len");
+      }
+      Tcap = std::max(Tcap, s.end - s.start);
+    }
+    g.d = d.d;
+    g.dh = d.dh;
+    g.nb = d.b;
+    g.elems = (long long)d.d * d.dh;
+    r = std::min(d.d, d.dh);
+    c = std::max(d.d, d.dh);
+    mat3 = (size_t)3 * d.b * g.elems;
+    nblk = std::max(1, std::min(256, (int)((g.elems + 2047) / 2048)));
+    lr_slots = ceil_div(d.dh, TSB::BN) * TSB::WAVES_N;
+    tiles = ceil_div(d.dh, TSA::BM) * ceil_div(d.d, TSA::BN);
+    tiles = std::max(tiles, ceil_div(d.d, TSA::BM) * ceil_div(d.dh, TSA::BN));
+    nsplit_max = choose_split(Tcap, tiles * 3 * d.b).n;
+
+    Bump sv;
+    s_n0 = sv.take((size_t)3 * d.b * g.maxrows() * 4);
+    s_wf = sv.take((size_t)(nupd + 1) * mat3 * 4);
+    s_wc = bf16 ? sv.take((size_t)(nupd + 1) * mat3 * 2) : s_wf;
+    s_main = d.prenorm ? sv.take((size_t)nupd * mat3 * 4) : 0;
+    s_d = sv.take((size_t)nupd * mat3 * 4);
+    s_mbar = sv.take((size_t)std::max(1, nupd) * d.b * 4);
+    s_u = muon ? sv.take((size_t)nupd * mat3 * 4) : 0;
+    s_g16 = muon ? sv.take((size_t)nupd * mat3 * nsz) : 0;
+    s_norms = sv.take((size_t)std::max(1, nupd) * 3 * d.b * 4);
+    s_xb = muon ? sv.take((size_t)nupd * std::max(1, S) * mat3 * nsz) : 0;
+    const size_t sq3 = (size_t)3 * d.b * r * r;
+    s_ab = muon ? sv.take((size_t)nupd * std::max(1, S) * sq3 * nsz) : 0;
+    s_bb = muon ? sv.take((size_t)nupd * std::max(1, S) * sq3 * nsz) : 0;
+    saved_bytes = sv.off + 256;
+
+    Bump sc;
+    for (int i = 0; i < 6; ++i) t_h[i] = sc.take((size_t)d.b * Tcap * d.dh * esz);
+    t_partial = sc.take((size_t)nsplit_max * mat3 * 4);
+    t_lrpart = sc.take((size_t)3 * lr_slots * d.b * Tcap * 4);
+    for (int i = 0; i < 2; ++i) t_xf[i] = sc.take(mat3 * 4);
+    t_xbtmp = sc.take(mat3 * nsz);
+    t_ss = sc.take((size_t)3 * d.b * nblk * 4);
+    t_dot = sc.take((size_t)3 * d.b * nblk * 4);
+    t_mdot = sc.take((size_t)3 * d.b * nblk * 4);
+    for (int i = 0; i < 2; ++i) t_gwhat[i] = sc.take(mat3 * 4);
+    t_gwcur = sc.take(mat3 * 4);
+    t_gmcarry = sc.take(mat3 * 4);
+    t_gc = sc.take(mat3 * esz);
+    for (int i = 0; i < 2; ++i) t_gxf[i] = sc.take(mat3 * 4);
+    for (int i = 0; i < 2; ++i) t_gxb[i] = sc.take(mat3 * nsz);
+    t_sg = sc.take(sq3 * nsz);
+    t_gas = sc.take(sq3 * nsz);
+    t_gn0 = sc.take((size_t)3 * d.b * g.maxrows() * 4);
+    scratch_bytes = sc.off + 256;
+    return 0;
+  }
+};
+
+inline char* align256(void* p) { return reinterpret_cast<char*>((reinterpret_cast<uintptr_t>(p) + 255) & ~uintptr_t(255)); }
+inline const char* align256(const void* p) {
+  return reinterpret_cast<const char*>((reinterpret_cast<uintptr_t>(p) + 255) & ~uintptr_t(255));
+}
+
+template <typename T, bool B_KC, int NT, int EPI>
+const char* row_gemm_name() {
+  static const std::string n = std::string("k_row_gemm<") + tname<T>() + (B_KC ? ",Bkc," : ",Bks,") + std::to_string(NT) +
+                               (EPI == EPI_STORE ? ",store>" : (EPI == EPI_AXPBY ? ",axpby>" : ",axpby_dual>"));
+  return n.c_str();
+}
+template <typename T, bool B_KC, int NT, int EPI>
+void launch_row_gemm(const char* site, const RowGemmParams<NT>& p, int batch, hipStream_t s) {
+  dim3 grid(ceil_div(p.M, TSA::BM), ceil_div(p.N, TSA::BN), batch);
+  double ksum = 0;
+  for (int t = 0; t < NT; ++t) ksum += p.t[t].K;
+  LACT_LAUNCH((row_gemm_name<T, B_KC, NT, EPI>()), site, 2.0 * p.M * p.N * ksum * batch,
+              (k_row_gemm<T, TSA, B_KC, NT, EPI>), grid, dim3(TSA::THREADS), s, p);
+}
+
+template <int NT>
+RowGemmParams<NT> row_params() {
+  RowGemmParams<NT> p;
+  memset(&p, 0, sizeof(p));
+  p.alpha = 1.f;
+  return p;
+}
+
+inline void set_term(RowGemmTerm& t, const void* A, int lda, long long bsA, const void* B, int ldb, long long bsB, int K) {
+  t.A = A; t.lda = lda; t.bsA = bsA; t.B = B; t.ldb = ldb; t.bsB = bsB; t.K = K;
+}
+inline void set_tr_term(TokenReduceTerm& t, const void* A, int lda, long long bsA, const void* B, int ldb, long long bsB) {
+  t.A = A; t.lda = lda; t.bsA = bsA; t.B = B; t.ldb = ldb; t.bsB = bsB;
+}
+
+// One Newton-Schulz iteration on n matrices held as [r, c] (always bf16 MFMA, fp32 iterate):
+//   A = X X^T;  B = b A + c A A;  X' = a X + B X        (ttt_operation.py:59-62)
+struct NsIter {
+  int n, r, c, nb_for_mask, mask, plain;
+  float ca, cb, cc;
+  const float* xf_in; const void* xb_in;           // X: fp32 iterate and its copy in the GEMM type
+  void* ab; void* bb;                              // A and B of this iteration (GEMM type)
+  float* xf_out; void* xb_out; float* u_out;       // X': fp32, GEMM type, and fp32 in the original orientation (each nullable)
+};
+// TN: GEMM operand type of the iteration (bf16 as in the reference, or fp32 for the exact mode)
+template <typename TN>
+void ns_iteration(const NsIter& I, hipStream_t s) {
+  const long long xe = (long long)I.r * I.c, se = (long long)I.r * I.r;
+  {
+    auto p = row_params<1>();
+    set_term(p.t[0], I.xb_in, I.c, xe, I.xb_in, I.c, xe, I.c);
+    p.M = I.r; p.N = I.r; p.out = I.ab; p.ldo = I.r; p.bso = se;
+    launch_row_gemm<TN, true, 1, EPI_STORE>("ns_gram", p, I.n, s);
+  }
+  {
+    auto p = row_params<1>();
+    set_term(p.t[0], I.ab, I.r, se, I.ab, I.r, se, I.r);
+    p.M = I.r; p.N = I.r; p.out = I.bb; p.ldo = I.r; p.bso = se;
+    p.aux = I.ab; p.ldaux = I.r; p.bsaux = se; p.alpha = I.cc; p.beta = I.cb;
+    launch_row_gemm<TN, true, 1, EPI_AXPBY>("ns_poly", p, I.n, s);
+  }
+  {
+    auto p = row_params<1>();
+    set_term(p.t[0], I.bb, I.r, se, I.xb_in, I.c, xe, I.r);
+    p.M = I.r; p.N = I.c; p.ldo = I.c; p.bso = xe;
+    p.aux = I.xf_in; p.ldaux = I.c; p.bsaux = xe; p.alpha = 1.f; p.beta = I.ca;
+    p.round_out_bf16 = I.plain;
+    p.out = I.xf_out; p.out_c = I.xb_out; p.out_t = I.u_out;
+    p.transpose_mask = I.mask; p.nb = I.nb_for_mask;
+    launch_row_gemm<TN, false, 1, EPI_AXPBY_F32_DUAL>("ns_next", p, I.n, s);
+  }
+}
+
+template <typename T, typename TN>
+struct Runner {
+  const Plan& P;
+  hipStream_t s;
+  char* sv;   // saved
+  char* sc;   // scratch
+  const lact_desc_t& d;
+  Runner(const Plan& p, void* saved, void* scratch, hipStream_t st)
+      : P(p), s(st), sv(align256(saved)), sc(align256(scratch)), d(p.d) {}
+
+  float* n0() const { return reinterpret_cast<float*>(sv + P.s_n0); }
+  float* wf(int ver) const { return reinterpret_cast<float*>(sv + P.s_wf) + (size_t)ver * P.mat3; }
+  T* wc(int ver) const { return reinterpret_cast<T*>(sv + P.s_wc) + (size_t)ver * P.mat3; }
+  T* wc(int ver, int j) const { return wc(ver) + (size_t)j * d.b * P.g.elems; }
+  // accumulator after `u` updates (pre-norm); main(0) is the initial weight
+  float* main_(int u) const { return u == 0 ? wf(0) : reinterpret_cast<float*>(sv + P.s_main) + (size_t)(u - 1) * P.mat3; }
+  float* dsave(int u) const { return reinterpret_cast<float*>(sv + P.s_d) + (size_t)u * P.mat3; }
+  float* mbar(int u) const { return reinterpret_cast<float*>(sv + P.s_mbar) + (size_t)u * d.b; }
+  float* usave(int u) const { return reinterpret_cast<float*>(sv + P.s_u) + (size_t)u * P.mat3; }
+  TN* g16(int u) const { return reinterpret_cast<TN*>(sv + P.s_g16) + (size_t)u * P.mat3; }
+  float* norms(int u) const { return reinterpret_cast<float*>(sv + P.s_norms) + (size_t)u * 3 * d.b; }
+  TN* xb(int u, int it) const { return reinterpret_cast<TN*>(sv + P.s_xb) + ((size_t)u * std::max(1, P.S) + it) * P.mat3; }
+  size_t sq3() const { return (size_t)3 * d.b * P.r * P.r; }
+  TN* ab(int u, int it) const { return reinterpret_cast<TN*>(sv + P.s_ab) + ((size_t)u * std::max(1, P.S) + it) * sq3(); }
+  TN* bb(int u, int it) const { return reinterpret_cast<TN*>(sv + P.s_bb) + ((size_t)u * std::max(1, P.S) + it) * sq3(); }
+  T* h(int i) const { return reinterpret_cast<T*>(sc + P.t_h[i]); }
+  template <typename U> U* scr(size_t off) const { return reinterpret_cast<U*>(sc + off); }
+
+  int tall_mask() const { return (P.g.tall(0) ? 1 : 0) | (P.g.tall(1) ? 2 : 0) | (P.g.tall(2) ? 4 : 0); }
+  long long hbs() const { return (long long)P.Tcap * d.dh; }
+
+  HiddenParams hidden_params(int T_, const void* X, int ldx, long long bsx, const void* Y, int ldy, long long bsy, int ver) const {
+    HiddenParams p;
+    memset(&p, 0, sizeof(p));
+    p.T = T_; p.d = d.d; p.dh = d.dh;
+    p.X = X; p.ldx = ldx; p.bsx = bsx;
+    p.Y = Y; p.ldy = ldy; p.bsy = bsy;
+    p.W0 = wc(ver, 0); p.W1 = wc(ver, 1); p.W2 = wc(ver, 2); p.bsw = P.g.elems;
+    p.bso = hbs();
+    p.Tcap = P.Tcap;
+    return p;
+  }
+
+  void token_reduce(const char* site, const TokenReduceJob (&jobs)[3], int tokens, Split sp) const {
+    TokenReduceParams p;
+    memset(&p, 0, sizeof(p));
+    for (int i = 0; i < 3; ++i) p.job[i] = jobs[i];
+    p.nb = d.b; p.tokens = tokens; p.split_len = sp.len;
+    p.partial = scr<float>(P.t_partial); p.mat_elems = P.g.elems;
+    dim3 grid(P.tiles, sp.n, 3 * d.b);
+    LACT_LAUNCH("k_token_reduce", site, 6.0 * tokens * d.d * d.dh * d.b * jobs[0].nterms, (k_token_reduce<T, TSA>), grid, dim3(TSA::THREADS), s, p);
+  }
+
+  RenormParams renorm_params(int u, int ver_prev) const {
+    RenormParams p;
+    memset(&p, 0, sizeof(p));
+    p.g = P.g;
+    const bool replace = P.muon && d.muon_replaces_weight;
+    p.base = d.prenorm ? main_(u) : wf(ver_prev);
+    p.cw = replace ? 0.f : 1.f;
+    p.u = P.muon ? usave(u) : dsave(u);
+    p.raw = replace ? dsave(u) : nullptr;
+    p.cr = replace ? 1.f : 0.f;
+    p.n0 = n0();
+    p.weight_norm = d.weight_norm;
+    return p;
+  }
+
+  // ------------------------------------------------------------------------------------------
+  int forward(const float* w0, const float* w1, const float* w2, const T* q, const T* k, const T* v, const float* lr0,
+              const float* lr1, const float* lr2, const float* mom, T* out, float* const w_out[3], float* const m_out[3]) {
+    const dim3 rowgrid(ceil_div(P.g.maxrows(), 4), 3 * d.b);
+    {
+      InitParams p;
+      p.g = P.g; p.w[0] = w0; p.w[1] = w1; p.w[2] = w2; p.n0 = n0(); p.wf = wf(0);
+      p.wc = P.bf16 ? (void*)wc(0) : nullptr;
+      LACT_LAUNCH("k_init_state", "k_init_state", 0.0, (k_init_state<T>), rowgrid, dim3(256), s, p);
+    }
+    int ver = 0, u = 0;
+    for (const auto& st : P.steps) {
+      const int T_ = st.end - st.start;
+      if (st.kind == LACT_APPLY) {
+        HiddenParams hp = hidden_params(T_, q + (size_t)st.start * d.q_ld, d.q_ld, d.q_bs, nullptr, 0, 0, ver);
+        hp.O0 = h(0);
+        dim3 grid(ceil_div(T_, TSA::BM), ceil_div(d.dh, TSA::BN), d.b);
+        LACT_LAUNCH("k_apply_hidden", "apply_hidden", 4.0 * T_ * d.d * d.dh * d.b, (k_apply_hidden<T, TSA>), grid, dim3(TSA::THREADS), s, hp);
+        auto p = row_params<1>();
+        set_term(p.t[0], h(0), d.dh, hbs(), wc(ver, 1), d.dh, P.g.elems, d.dh);
+        p.M = T_; p.N = d.d; p.out = out + (size_t)st.out_start * d.o_ld; p.ldo = d.o_ld; p.bso = d.o_bs;
+        launch_row_gemm<T, true, 1, EPI_STORE>("apply_out", p, d.b, s);
+        continue;
+      }
+      // ---- update
+      const T* kc = k + (size_t)st.start * d.k_ld;
+      const T* vc = v + (size_t)st.start * d.v_ld;
+      {
+        HiddenParams hp = hidden_params(T_, kc, d.k_ld, d.k_bs, vc, d.v_ld, d.v_bs, ver);
+        hp.lr0 = lr0 + st.start; hp.lr1 = lr1 + st.start; hp.lr2 = lr2 + st.start; hp.bslr = d.kv_len;
+        hp.O0 = h(0); hp.O1 = h(1); hp.O2 = h(2);
+        dim3 grid(ceil_div(T_, TSA::BM), ceil_div(d.dh, TSA::BN), d.b);
+        LACT_LAUNCH("k_update_hidden", "update_hidden", 6.0 * T_ * d.d * d.dh * d.b, (k_update_hidden<T, TSA>), grid, dim3(TSA::THREADS), s, hp);
+      }
+      const Split sp = choose_split(T_, P.tiles * 3 * d.b);
+      {
+        TokenReduceJob jobs[3];
+        memset(jobs, 0, sizeof(jobs));
+        jobs[0].nterms = jobs[1].nterms = jobs[2].nterms = 1;
+        jobs[0].M = d.dh; jobs[0].N = d.d;
+        set_tr_term(jobs[0].t[0], h(0), d.dh, hbs(), kc, d.k_ld, d.k_bs);
+        jobs[1].M = d.d; jobs[1].N = d.dh;
+        set_tr_term(jobs[1].t[0], vc, d.v_ld, d.v_bs, h(1), d.dh, hbs());
+        jobs[2].M = d.dh; jobs[2].N = d.d;
+        set_tr_term(jobs[2].t[0], h(2), d.dh, hbs(), kc, d.k_ld, d.k_bs);
+        token_reduce("update_dw", jobs, T_, sp);
+      }
+      if (P.momentum) LACT_LAUNCH("k_momentum_mean", "k_momentum_mean", 0.0, k_momentum_mean, dim3(d.b), dim3(256), s, mom, (long long)d.kv_len, st.start, T_, mbar(u));
+      {
+        MomentumPrepParams p;
+        memset(&p, 0, sizeof(p));
+        p.g = P.g; p.partial = scr<float>(P.t_partial); p.nsplit = sp.n;
+        p.m_prev = (P.momentum && u > 0) ? dsave(u - 1) : nullptr;
+        p.mbar = P.momentum ? mbar(u) : nullptr;
+        p.d_out = dsave(u);
+        p.g16 = P.muon ? g16(u) : nullptr;
+        p.ss_part = scr<float>(P.t_ss);
+        p.round_partial_bf16 = P.bf16;
+        LACT_LAUNCH("k_momentum_prep", "k_momentum_prep", 0.0, (k_momentum_prep<TN>), dim3(P.nblk, 3 * d.b), dim3(256), s, p);
+      }
+      if (P.muon) {
+        NsScaleParams p;
+        memset(&p, 0, sizeof(p));
+        p.g = P.g; p.g16 = g16(u); p.ss_part = scr<float>(P.t_ss); p.nparts = P.nblk; p.norms = norms(u);
+        p.xf = scr<float>(P.t_xf[0]); p.xb = xb(u, 0);
+        p.u = P.S == 0 ? usave(u) : nullptr;
+        p.plain_bf16 = d.ns_mode == LACT_NS_PLAIN_BF16;
+        LACT_LAUNCH("k_ns_scale", "k_ns_scale", 0.0, (k_ns_scale<TN>), dim3(P.nblk, 3 * d.b), dim3(256), s, p);
+        for (int it = 0; it < P.S; ++it) {
+          const bool last = it + 1 == P.S;
+          NsIter I;
+          I.n = 3 * d.b; I.r = P.r; I.c = P.c; I.nb_for_mask = d.b; I.mask = tall_mask(); I.plain = d.ns_mode == LACT_NS_PLAIN_BF16;
+          I.ca = P.coeffs[3 * it]; I.cb = P.coeffs[3 * it + 1]; I.cc = P.coeffs[3 * it + 2];
+          I.xf_in = scr<float>(P.t_xf[it & 1]); I.xb_in = xb(u, it);
+          I.ab = ab(u, it); I.bb = bb(u, it);
+          I.xf_out = last ? nullptr : scr<float>(P.t_xf[(it + 1) & 1]);
+          I.xb_out = last ? (void*)scr<TN>(P.t_xbtmp) : (void*)xb(u, it + 1);
+          I.u_out = last ? usave(u) : nullptr;
+          ns_iteration<TN>(I, s);
+        }
+      }
+      {
+        RenormParams p = renorm_params(u, ver);
+        p.main_out = d.prenorm ? main_(u + 1) : nullptr;
+        p.wf_out = wf(ver + 1);
+        p.wc_out = P.bf16 ? (void*)wc(ver + 1) : nullptr;
+        LACT_LAUNCH("k_update_renorm", "k_update_renorm", 0.0, (k_update_renorm<T>), rowgrid, dim3(256), s, p);
+      }
+      ++ver;
+      ++u;
+    }
+    const dim3 eg((unsigned)((P.g.elems + 255) / 256), 3 * d.b);
+    if (w_out && (w_out[0] || w_out[1] || w_out[2]))
+      LACT_LAUNCH("k_unpack3", "k_unpack3", 0.0, k_unpack3, eg, dim3(256), s, wf(ver), P.g.elems, d.b, w_out[0], w_out[1], w_out[2]);
+    if (m_out && (m_out[0] || m_out[1] || m_out[2])) {
+      if (u > 0 && P.momentum)
+        LACT_LAUNCH("k_unpack3", "k_unpack3", 0.0, k_unpack3, eg, dim3(256), s, dsave(u - 1), P.g.elems, d.b, m_out[0], m_out[1], m_out[2]);
+      else
+        for (int j = 0; j < 3; ++j)
+          if (m_out[j]) LACT_LAUNCH("k_fill_f32", "k_fill_f32", 0.0, k_fill_f32, dim3((unsigned)((d.b * P.g.elems + 255) / 256)), dim3(256), s, m_out[j], 0.f, (long long)d.b * P.g.elems);
+    }
+    LACT_CHECK_LAUNCH();
+    return 0;
+  }
+
+  // ------------------------------------------------------------------------------------------
+  static bool overlaps(std::vector<std::pair<int, int>>& seen, int a, int b) {
+    bool hit = false;
+    for (auto& iv : seen) hit = hit || (a < iv.second && iv.first < b);
+    seen.emplace_back(a, b);
+    return hit;
+  }
+
+  int backward(const T* q, const T* k, const T* v, const float* lr0, const float* lr1, const float* lr2, const float* mom,
+               const T* dout, const float* const dwf[3], float* dw0, float* dw1, float* dw2, T* dq, T* dk, T* dv, float* dlr0,
+               float* dlr1, float* dlr2, float* dmom) {
+    (void)mom;
+    const dim3 rowgrid(ceil_div(P.g.maxrows(), 4), 3 * d.b);
+    const dim3 eg((unsigned)((P.g.elems + 255) / 256), 3 * d.b);
+    const dim3 flat((unsigned)((P.mat3 + 255) / 256));
+    float* gwcur = scr<float>(P.t_gwcur);
+    float* gn0 = scr<float>(P.t_gn0);
+    float* gmcarry = scr<float>(P.t_gmcarry);
+    float* partial = scr<float>(P.t_partial);
+    const long long gn0_n = (long long)3 * d.b * P.g.maxrows();
+    LACT_LAUNCH("k_fill_f32", "k_fill_f32", 0.0, k_fill_f32, dim3((unsigned)((gn0_n + 255) / 256)), dim3(256), s, gn0, 0.f, gn0_n);
+    LACT_LAUNCH("k_pack3", "k_pack3", 0.0, k_pack3, eg, dim3(256), s, gwcur, P.g.elems, d.b, dwf ? dwf[0] : nullptr, dwf ? dwf[1] : nullptr,
+                       dwf ? dwf[2] : nullptr);
+    std::vector<std::pair<int, int>> seen_q, seen_kv;
+    int ver = P.nupd, u = P.nupd;
+    int carry_main = -1;       // index of the gwhat buffer holding the accumulator's gradient (pre-norm)
+    bool gm_valid = false;     // gmcarry holds d loss / d (momentum state after update u-1)
+    for (int si = (int)P.steps.size() - 1; si >= 0; --si) {
+      const lact_step_t& st = P.steps[si];
+      const int T_ = st.end - st.start;
+      const Split sp = choose_split(T_, P.tiles * 3 * d.b);
+      if (st.kind == LACT_APPLY) {
+        const T* qc = q + (size_t)st.start * d.q_ld;
+        const T* gc = dout + (size_t)st.out_start * d.do_ld;
+        HiddenParams hp = hidden_params(T_, qc, d.q_ld, d.q_bs, gc, d.do_ld, d.do_bs, ver);
+        hp.O0 = h(0); hp.O1 = h(1); hp.O2 = h(2);
+        dim3 grid(ceil_div(T_, TSA::BM), ceil_div(d.dh, TSA::BN), d.b);
+        LACT_LAUNCH("k_apply_bwd_hidden", "apply_bwd_hidden", 6.0 * T_ * d.d * d.dh * d.b, (k_apply_bwd_hidden<T, TSA>), grid, dim3(TSA::THREADS), s, hp);
+        {  // dq = gY0 W0 + gY2 W2
+          auto p = row_params<2>();
+          set_term(p.t[0], h(1), d.dh, hbs(), wc(ver, 0), d.d, P.g.elems, d.dh);
+          set_term(p.t[1], h(2), d.dh, hbs(), wc(ver, 2), d.d, P.g.elems, d.dh);
+          p.M = T_; p.N = d.d; p.out = dq + (size_t)st.start * d.d; p.ldo = d.d; p.bso = (long long)d.q_len * d.d;
+          p.accumulate = overlaps(seen_q, st.start, st.end);
+          launch_row_gemm<T, false, 2, EPI_STORE>("apply_bwd_dq", p, d.b, s);
+        }
+        TokenReduceJob jobs[3];
+        memset(jobs, 0, sizeof(jobs));
+        jobs[0].nterms = jobs[1].nterms = jobs[2].nterms = 1;
+        jobs[0].M = d.dh; jobs[0].N = d.d;
+        set_tr_term(jobs[0].t[0], h(1), d.dh, hbs(), qc, d.q_ld, d.q_bs);
+        jobs[1].M = d.d; jobs[1].N = d.dh;
+        set_tr_term(jobs[1].t[0], gc, d.do_ld, d.do_bs, h(0), d.dh, hbs());
+        jobs[2].M = d.dh; jobs[2].N = d.d;
+        set_tr_term(jobs[2].t[0], h(2), d.dh, hbs(), qc, d.q_ld, d.q_bs);
+        token_reduce("apply_bwd_dw", jobs, T_, sp);
+        LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, gwcur, gwcur, 1.f, partial, sp.n, (long long)P.mat3);
+        continue;
+      }
+      // ---- update u-1: weights ver-1 -> ver
+      --u;
+      const int vprev = ver - 1;
+      const int gw_idx = carry_main == 0 ? 1 : 0;
+      float* gwhat = scr<float>(P.t_gwhat[gw_idx]);
+      int cur = 0;  // which gxf/gxb buffer holds the running Newton-Schulz gradient
+      {
+        RenormParams p = renorm_params(u, vprev);
+        p.gy = gwcur;
+        p.carry_in = (d.prenorm && carry_main >= 0) ? scr<float>(P.t_gwhat[carry_main]) : nullptr;
+        p.gw_hat = gwhat;
+        p.gn0 = gn0;
+        if (P.muon) { p.gxf = scr<float>(P.t_gxf[0]); p.gxb = scr<TN>(P.t_gxb[0]); }
+        LACT_LAUNCH("k_renorm_bwd", "k_renorm_bwd", 0.0, (k_renorm_bwd<TN>), rowgrid, dim3(256), s, p);
+      }
+      if (d.prenorm) carry_main = gw_idx;
+      if (P.muon) {
+        const int n = 3 * d.b, r = P.r, c = P.c;
+        const long long xe = (long long)r * c, se = (long long)r * r;
+        TN* sg = scr<TN>(P.t_sg);
+        TN* gas = scr<TN>(P.t_gas);
+        for (int it = P.S - 1; it >= 0; --it) {
+          const float ca = P.coeffs[3 * it], cb = P.coeffs[3 * it + 1], cc = P.coeffs[3 * it + 2];
+          TN* gb = scr<TN>(P.t_gxb[cur]);
+          float* gf = scr<float>(P.t_gxf[cur]);
+          {  // Sg = G X^T + X G^T
+            auto p = row_params<2>();
+            set_term(p.t[0], gb, c, xe, xb(u, it), c, xe, c);
+            set_term(p.t[1], xb(u, it), c, xe, gb, c, xe, c);
+            p.M = r; p.N = r; p.out = sg; p.ldo = r; p.bso = se;
+            launch_row_gemm<TN, true, 2, EPI_STORE>("ns_bwd_sg", p, n, s);
+          }
+          {  // gA + gA^T = b Sg + c (Sg A + A Sg)
+            auto p = row_params<2>();
+            set_term(p.t[0], sg, r, se, ab(u, it), r, se, r);
+            set_term(p.t[1], ab(u, it), r, se, sg, r, se, r);
+            p.M = r; p.N = r; p.out = gas; p.ldo = r; p.bso = se;
+            p.aux = sg; p.ldaux = r; p.bsaux = se; p.alpha = cc; p.beta = cb;
+            launch_row_gemm<TN, true, 2, EPI_AXPBY>("ns_bwd_ga", p, n, s);
+          }
+          {  // gX = a G + B G + (gA + gA^T) X
+            auto p = row_params<2>();
+            set_term(p.t[0], bb(u, it), r, se, gb, c, xe, r);
+            set_term(p.t[1], gas, r, se, xb(u, it), c, xe, r);
+            p.M = r; p.N = c; p.ldo = c; p.bso = xe;
+            p.aux = gf; p.ldaux = c; p.bsaux = xe; p.alpha = 1.f; p.beta = ca;
+            p.out = scr<float>(P.t_gxf[cur ^ 1]);
+            p.out_c = scr<TN>(P.t_gxb[cur ^ 1]);
+            launch_row_gemm<TN, false, 2, EPI_AXPBY_F32_DUAL>("ns_bwd_gx", p, n, s);
+          }
+          cur ^= 1;
+        }
+        NsDotParams dp;
+        dp.g = P.g; dp.gx0 = scr<float>(P.t_gxf[cur]); dp.g16 = g16(u); dp.dot_part = scr<float>(P.t_dot);
+        LACT_LAUNCH("k_ns_bwd_dot", "k_ns_bwd_dot", 0.0, (k_ns_bwd_dot<TN>), dim3(P.nblk, 3 * d.b), dim3(256), s, dp);
+      }
+      {
+        GradPrepParams p;
+        memset(&p, 0, sizeof(p));
+        p.g = P.g; p.muon = P.muon;
+        p.gx0 = scr<float>(P.t_gxf[cur]); p.g16 = P.muon ? (const void*)g16(u) : nullptr; p.norms = norms(u);
+        p.dot_part = scr<float>(P.t_dot); p.nparts = P.nblk;
+        p.gw_hat = gwhat; p.cr = (P.muon && d.muon_replaces_weight) ? 1.f : 0.f;
+        p.gm_carry = P.momentum ? gmcarry : nullptr; p.carry_valid = gm_valid;
+        p.m_prev = (P.momentum && u > 0) ? dsave(u - 1) : nullptr;
+        p.mbar = P.momentum ? mbar(u) : nullptr;
+        p.gc = scr<T>(P.t_gc);
+        p.mdot_part = scr<float>(P.t_mdot);
+        LACT_LAUNCH("k_grad_prep", "k_grad_prep", 0.0, (k_grad_prep<T, TN>), dim3(P.nblk, 3 * d.b), dim3(256), s, p);
+        if (P.momentum) {
+          gm_valid = true;
+          if (u > 0)
+            LACT_LAUNCH("k_momentum_grad", "k_momentum_grad", 0.0, k_momentum_grad, dim3(d.b), dim3(256), s, scr<float>(P.t_mdot), P.nblk, d.b, dmom,
+                               (long long)d.kv_len, st.start, T_);
+        }
+      }
+      const T* kc = k + (size_t)st.start * d.k_ld;
+      const T* vc = v + (size_t)st.start * d.v_ld;
+      T* gcm = scr<T>(P.t_gc);
+      T* g0 = gcm; T* g1 = gcm + (size_t)d.b * P.g.elems; T* g2 = gcm + (size_t)2 * d.b * P.g.elems;
+      {
+        HiddenParams hp = hidden_params(T_, kc, d.k_ld, d.k_bs, vc, d.v_ld, d.v_bs, vprev);
+        hp.lr0 = lr0 + st.start; hp.lr1 = lr1 + st.start; hp.lr2 = lr2 + st.start; hp.bslr = d.kv_len;
+        hp.G0 = g0; hp.G1 = g1; hp.G2 = g2;
+        hp.O0 = h(0); hp.O1 = h(1); hp.O2 = h(2); hp.O3 = h(3); hp.O4 = h(4); hp.O5 = h(5);
+        hp.lrpart = scr<float>(P.t_lrpart);
+        hp.lrpart_stride = (long long)d.b * P.Tcap;
+        hp.lrpart_mat_stride = (long long)P.lr_slots * d.b * P.Tcap;
+        dim3 grid(ceil_div(T_, TSB::BM), ceil_div(d.dh, TSB::BN), d.b);
+        LACT_LAUNCH("k_update_bwd_hidden", "update_bwd_hidden", 12.0 * T_ * d.d * d.dh * d.b, (k_update_bwd_hidden<T, TSB>), grid, dim3(TSB::THREADS), s, hp);
+      }
+      const bool acc_kv = overlaps(seen_kv, st.start, st.end);
+      {  // dk = (dgate*lr0) G0 + (dh2*lr2) G2 + gG W0 + gH2 W2
+        auto p = row_params<4>();
+        set_term(p.t[0], h(3), d.dh, hbs(), g0, d.d, P.g.elems, d.dh);
+        set_term(p.t[1], h(5), d.dh, hbs(), g2, d.d, P.g.elems, d.dh);
+        set_term(p.t[2], h(0), d.dh, hbs(), wc(vprev, 0), d.d, P.g.elems, d.dh);
+        set_term(p.t[3], h(2), d.dh, hbs(), wc(vprev, 2), d.d, P.g.elems, d.dh);
+        p.M = T_; p.N = d.d; p.out = dk + (size_t)st.start * d.d; p.ldo = d.d; p.bso = (long long)d.kv_len * d.d;
+        p.accumulate = acc_kv;
+        launch_row_gemm<T, false, 4, EPI_STORE>("update_bwd_dk", p, d.b, s);
+      }
+      {  // dv = (hidden*lr1) G1^T + gDH W1^T
+        auto p = row_params<2>();
+        set_term(p.t[0], h(4), d.dh, hbs(), g1, d.dh, P.g.elems, d.dh);
+        set_term(p.t[1], h(1), d.dh, hbs(), wc(vprev, 1), d.dh, P.g.elems, d.dh);
+        p.M = T_; p.N = d.d; p.out = dv + (size_t)st.start * d.d; p.ldo = d.d; p.bso = (long long)d.kv_len * d.d;
+        p.accumulate = acc_kv;
+        launch_row_gemm<T, true, 2, EPI_STORE>("update_bwd_dv", p, d.b, s);
+      }
+      {
+        TokenReduceJob jobs[3];
+        memset(jobs, 0, sizeof(jobs));
+        jobs[0].nterms = jobs[1].nterms = jobs[2].nterms = 1;
+        jobs[0].M = d.dh; jobs[0].N = d.d;
+        set_tr_term(jobs[0].t[0], h(0), d.dh, hbs(), kc, d.k_ld, d.k_bs);
+        jobs[1].M = d.d; jobs[1].N = d.dh;
+        set_tr_term(jobs[1].t[0], vc, d.v_ld, d.v_bs, h(1), d.dh, hbs());
+        jobs[2].M = d.dh; jobs[2].N = d.d;
+        set_tr_term(jobs[2].t[0], h(2), d.dh, hbs(), kc, d.k_ld, d.k_bs);
+        token_reduce("update_bwd_dw", jobs, T_, sp);
+        const float pass = d.prenorm ? 0.f : ((P.muon && d.muon_replaces_weight) ? 0.f : 1.f);
+        LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, gwcur, gwhat, pass, partial, sp.n, (long long)P.mat3);
+      }
+      LACT_LAUNCH("k_lr_reduce", "k_lr_reduce", 0.0, k_lr_reduce, dim3(ceil_div(T_, 256), d.b, 3), dim3(256), s, scr<float>(P.t_lrpart),
+                         (long long)P.lr_slots * d.b * P.Tcap, (long long)d.b * P.Tcap, P.lr_slots, P.Tcap, dlr0, dlr1, dlr2,
+                         (long long)d.kv_len, st.start, T_);
+      --ver;
+    }
+    {
+      FinishParams p;
+      p.g = P.g; p.gw = gwcur;
+      p.carry = (d.prenorm && carry_main >= 0) ? scr<float>(P.t_gwhat[carry_main]) : nullptr;
+      p.gn0 = gn0; p.n0 = n0(); p.w_init = wf(0);
+      p.through_norms = d.detach_norms ? 0 : 1;
+      p.out[0] = dw0; p.out[1] = dw1; p.out[2] = dw2;
+      LACT_LAUNCH("k_finish_weight_grads", "k_finish_weight_grads", 0.0, k_finish_weight_grads, rowgrid, dim3(256), s, p);
+    }
+    LACT_CHECK_LAUNCH();
+    return 0;
+  }
+};
+
+int check_ptrs(std::initializer_list<const void*> ps, const char* what) {
+  for (const void* p : ps)
+    if (!p) return fail(std::string("null pointer: ") + what);
+  return 0;
+}
+
+}  // namespace
+
+// ---- standalone Newton-Schulz ---------------------------------------------------------------
+namespace {
+struct NsPlan {
+  MatGeom g;
+  int r, c, nblk;
+  size_t o_g16, o_ss, o_norm, o_xf[2], o_xb[2], o_ab, o_bb, bytes;
+  void build(int n, int rows, int cols) {
+    // one "matrix kind" (index 0) of shape [rows, cols]: d = cols, dh = rows
+    g.d = cols; g.dh = rows; g.nb = n; g.elems = (long long)rows * cols;
+    r = std::min(rows, cols); c = std::max(rows, cols);
+    nblk = std::max(1, std::min(256, (int)((g.elems + 2047) / 2048)));
+    Bump b;
+    const size_t e = (size_t)n * g.elems;
+    o_g16 = b.take(e * 4); o_ss = b.take((size_t)n * nblk * 4); o_norm = b.take((size_t)n * 4);
+    o_xf[0] = b.take(e * 4); o_xf[1] = b.take(e * 4); o_xb[0] = b.take(e * 4); o_xb[1] = b.take(e * 4);
+    o_ab = b.take((size_t)n * r * r * 4); o_bb = b.take((size_t)n * r * r * 4);
+    bytes = b.off + 256;
+  }
+};
+}  // namespace
+
+namespace {
+template <typename TN>
+int newton_schulz_t(int32_t n, int32_t rows, int32_t cols, const float* gin, float* out, int32_t steps, const float* coeffs,
+                    int32_t ns_mode, void* workspace, hipStream_t s) {
+  const int plain_bf16 = ns_mode == LACT_NS_PLAIN_BF16;
+  NsPlan P;
+  P.build(n, rows, cols);
+  char* ws = align256(workspace);
+  // MatGeom treats index 0 as [dh, d] = [rows, cols]; launch with grid.y = n so z / nb == 0 throughout.
+  MomentumPrepParams mp;
+  memset(&mp, 0, sizeof(mp));
+  mp.g = P.g; mp.partial = gin; mp.nsplit = 1; mp.d_out = reinterpret_cast<float*>(ws + P.o_xf[1]);
+  mp.g16 = ws + P.o_g16; mp.ss_part = reinterpret_cast<float*>(ws + P.o_ss);
+  // partial is indexed [s][3*nb][elems] with z < nb: the layout of gin ([n][elems]) matches for s = 0
+  LACT_LAUNCH("k_momentum_prep", "k_momentum_prep", 0.0, (k_momentum_prep<TN>), dim3(P.nblk, n), dim3(256), s, mp);
+  NsScaleParams sp;
+  memset(&sp, 0, sizeof(sp));
+  sp.g = P.g; sp.g16 = mp.g16; sp.ss_part = mp.ss_part; sp.nparts = P.nblk; sp.norms = reinterpret_cast<float*>(ws + P.o_norm);
+  sp.xf = reinterpret_cast<float*>(ws + P.o_xf[0]); sp.xb = ws + P.o_xb[0];
+  sp.u = steps == 0 ? out : nullptr; sp.plain_bf16 = plain_bf16;
+  LACT_LAUNCH("k_ns_scale", "k_ns_scale", 0.0, (k_ns_scale<TN>), dim3(P.nblk, n), dim3(256), s, sp);
+  for (int it = 0; it < steps; ++it) {
+    const bool last = it + 1 == steps;
+    NsIter I;
+    I.n = n; I.r = P.r; I.c = P.c; I.nb_for_mask = n; I.mask = P.g.tall(0) ? 1 : 0; I.plain = plain_bf16;
+    I.ca = coeffs[3 * it]; I.cb = coeffs[3 * it + 1]; I.cc = coeffs[3 * it + 2];
+    I.xf_in = reinterpret_cast<float*>(ws + P.o_xf[it & 1]);
+    I.xb_in = ws + P.o_xb[it & 1];
+    I.ab = ws + P.o_ab; I.bb = ws + P.o_bb;
+    I.xf_out = last ? nullptr : reinterpret_cast<float*>(ws + P.o_xf[(it + 1) & 1]);
+    I.xb_out = last ? nullptr : ws + P.o_xb[(it + 1) & 1];
+    I.u_out = last ? out : nullptr;
+    ns_iteration<TN>(I, s);
+  }
+  LACT_CHECK_LAUNCH();
+  return 0;
+}
+}  // namespace
+
+
+extern "C" {
+
+const char* lact_last_error(void) { return g_err.c_str(); }
+int lact_version(void) { return 1; }
+
+int lact_profile_enable(int on) {
+  g_prof.clear();
+  g_prof.on = on != 0;
+  return 0;
+}
+
+int lact_profile_report(char* buf, size_t cap) {
+  if (!buf || cap == 0) return fail("null report buffer");
+  hipError_t e = hipDeviceSynchronize();
+  if (e != hipSuccess) return fail(std::string("synchronize failed: ") + hipGetErrorString(e));
+  struct Agg { std::string kernel, site; long n = 0; double ms = 0, flops = 0; };
+  std::vector<Agg> aggs;
+  for (auto& r : g_prof.recs) {
+    float ms = 0.f;
+    if (hipEventElapsedTime(&ms, r.e0, r.e1) != hipSuccess) continue;
+    Agg* a = nullptr;
+    for (auto& x : aggs)
+      if (x.kernel == r.kernel && x.site == r.site) a = &x;
+    if (!a) {
+      aggs.push_back(Agg{r.kernel, r.site});
+      a = &aggs.back();
+    }
+    a->n += 1;
+    a->ms += ms;
+    a->flops += r.flops;
+  }
+  std::string out = "[";
+  for (size_t i = 0; i < aggs.size(); ++i) {
+    char line[512];
+    snprintf(line, sizeof(line), "%s{\"kernel\": \"%s\", \"site\": \"%s\", \"launches\": %ld, \"ms\": %.6f, \"flops\": %.6e}",
+             i ? ", " : "", aggs[i].kernel.c_str(), aggs[i].site.c_str(), aggs[i].n, aggs[i].ms, aggs[i].flops);
+    out += line;
+  }
+  out += "]";
+  g_prof.clear();
+  if (out.size() + 1 > cap) return fail("report buffer too small");
+  memcpy(buf, out.c_str(), out.size() + 1);
+  return 0;
+}
+
+int lact_query_sizes(const lact_desc_t* desc, size_t* saved_bytes, size_t* scratch_bytes) {
+  Plan P;
+  if (P.build(desc)) return -1;
+  if (saved_bytes) *saved_bytes = P.saved_bytes;
+  if (scratch_bytes) *scratch_bytes = P.scratch_bytes;
+  return 0;
+}
+
+int lact_forward(const lact_desc_t* desc, const float* w0, const float* w1, const float* w2, const void* q, const void* k,
+                 const void* v, const float* lr0, const float* lr1, const float* lr2, const float* momentum, void* out,
+                 float* const w_out[3], float* const m_out[3], void* saved, void* scratch, void* stream) {
+  Plan P;
+  if (P.build(desc)) return -1;
+  if (check_ptrs({w0, w1, w2, q, out, saved, scratch}, "forward tensors")) return -1;
+  if (P.nupd > 0 && check_ptrs({k, v, lr0, lr1, lr2}, "k, v, lr")) return -1;
+  if (P.nupd > 0 && P.momentum && !momentum) return fail("use_momentum set but momentum is null");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+#define LACT_FWD(T_, TN_)                                                                                           \
+  {                                                                                                                 \
+    Runner<T_, TN_> R(P, saved, scratch, s);                                                                        \
+    return R.forward(w0, w1, w2, (const T_*)q, (const T_*)k, (const T_*)v, lr0, lr1, lr2, momentum, (T_*)out, w_out, \
+                     m_out);                                                                                        \
+  }
+  const bool ns32 = P.d.ns_mode == LACT_NS_FP32;
+  if (P.bf16 && !ns32) LACT_FWD(uint16_t, uint16_t)
+  if (P.bf16 && ns32) LACT_FWD(uint16_t, float)
+  if (!ns32) LACT_FWD(float, uint16_t)
+  LACT_FWD(float, float)
+#undef LACT_FWD
+}
+
+int lact_backward(const lact_desc_t* desc, const void* q, const void* k, const void* v, const float* lr0, const float* lr1,
+                  const float* lr2, const float* momentum, const void* dout, const float* const dw_final[3], const void* saved,
+                  void* scratch, float* dw0, float* dw1, float* dw2, void* dq, void* dk, void* dv, float* dlr0, float* dlr1,
+                  float* dlr2, float* dmomentum, void* stream) {
+  Plan P;
+  if (P.build(desc)) return -1;
+  if (check_ptrs({q, dout, saved, scratch, dw0, dw1, dw2, dq}, "backward tensors")) return -1;
+  if (P.nupd > 0 && check_ptrs({k, v, lr0, lr1, lr2, dk, dv, dlr0, dlr1, dlr2}, "k, v, lr and their gradients")) return -1;
+  if (P.nupd > 0 && P.momentum && (!momentum || !dmomentum)) return fail("use_momentum set but momentum or dmomentum is null");
+  const int al = P.bf16 ? 8 : 4;
+  if (P.d.do_ld % al || P.d.do_bs % al || P.d.do_ld < P.d.d) return fail("dout strides must keep 16-byte alignment");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+#define LACT_BWD(T_, TN_)                                                                                            \
+  {                                                                                                                  \
+    Runner<T_, TN_> R(P, const_cast<void*>(saved), scratch, s);                                                      \
+    return R.backward((const T_*)q, (const T_*)k, (const T_*)v, lr0, lr1, lr2, momentum, (const T_*)dout, dw_final,  \
+                      dw0, dw1, dw2, (T_*)dq, (T_*)dk, (T_*)dv, dlr0, dlr1, dlr2, dmomentum);                        \
+  }
+  const bool ns32 = P.d.ns_mode == LACT_NS_FP32;
+  if (P.bf16 && !ns32) LACT_BWD(uint16_t, uint16_t)
+  if (P.bf16 && ns32) LACT_BWD(uint16_t, float)
+  if (!ns32) LACT_BWD(float, uint16_t)
+  LACT_BWD(float, float)
+#undef LACT_BWD
+}
+
+size_t lact_newton_schulz_workspace_bytes(int32_t n, int32_t rows, int32_t cols, int32_t steps) {
+  (void)steps;
+  if (n <= 0 || rows <= 0 || cols <= 0) return 0;
+  NsPlan P;
+  P.build(n, rows, cols);
+  return P.bytes;
+}
+
+int lact_newton_schulz(int32_t n, int32_t rows, int32_t cols, const float* gin, float* out, int32_t steps, const float* coeffs,
+                       int32_t ns_mode, void* workspace, void* stream) {
+  if (n <= 0 || rows <= 0 || cols <= 0 || n > 65535) return fail("bad Newton-Schulz shape");
+  if (rows % 8 || cols % 8) return fail("rows and cols must be multiples of 8");
+  if (steps < 0 || steps > 64 || (steps > 0 && !coeffs)) return fail("bad Newton-Schulz steps");
+  if (ns_mode < 0 || ns_mode > 2) return fail("ns_mode must be 0, 1 or 2");
+  if (!gin || !out || !workspace) return fail("null pointer: newton_schulz");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (ns_mode == LACT_NS_FP32) return newton_schulz_t<float>(n, rows, cols, gin, out, steps, coeffs, ns_mode, workspace, s);
+  return newton_schulz_t<uint16_t>(n, rows, cols, gin, out, steps, coeffs, ns_mode, workspace, s);
+}
+
+}  // extern "C"
