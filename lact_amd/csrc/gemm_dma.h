@@ -1,0 +1,252 @@
+// bf16 GEMM main loop for gfx950 with asynchronous global->LDS copies and a multi-stage ring.
+//
+//   for every phase p:   acc[p][j] += A_p (BM x K_p)  *  B_pj (BN x K_p)^T        j < NB
+//
+// Every operand is K-contiguous (element (r,k) at base[r*ld + k]).  A block is 4 waves; BK = 64.
+// One stage of the ring holds the A tile and up to NB B tiles of one K-step; tiles are copied with
+// global_load_lds_dwordx4 (16 bytes per lane straight into LDS, no VGPR staging), so STAGES-1 K-steps
+// of loads stay in flight across the MFMA work -- what hides the ~1.5 us memory latency that a
+// register-staged, one-step-ahead prefetch leaves exposed.  All phases run through one flat
+// iteration space, so the ring never drains between phases.
+//
+// LDS tile layout: [row][64 bf16] = 128 B per row, unpadded (a wave's 64 lanes x 16 B land as one
+// contiguous 1 KiB, 8 rows).  The 16-byte k-granule j of row r is stored at slot j ^ ((r >> 1) & 7):
+// ds_read_b128 serves 16 lanes per clock, and 16 consecutive rows then cover all 64 banks.
+#pragma once
+#include "gemm_core.h"
+
+// Optional in-kernel timestamps (defined only by timing experiments; expands to nothing in the library).
+#ifndef LACT_TS
+#define LACT_TS(i)
+#endif
+
+namespace lact {
+
+__device__ __forceinline__ uint32_t lds_addr(const void* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+}
+
+// 16 bytes per lane from global memory (uniform 64-bit base + per-lane 32-bit byte offset) to LDS: lane i
+// lands at lds_base + 16*i (lds_base wave-uniform).  No vector-ALU work per copy: bases live in SGPRs.
+__device__ __forceinline__ void dma16(const void* sbase, uint32_t voff, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t" ::"s"(lds_base), "v"(voff), "s"(sbase)
+               : "memory", "m0");
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+struct DmaOperand {
+  const uint16_t* base;  // first row of this block's tile
+  int ld;
+  int rows;              // valid rows from base on (may exceed the tile)
+};
+
+// One phase: acc[j] += A * B_j^T over K, j < nb.
+template <int NBMAX>
+struct DmaPhase {
+  DmaOperand a;
+  DmaOperand b[NBMAX];
+  int nb;
+  int K;
+};
+
+constexpr int DMA_BK = 64;
+
+// Loader-wave addressing of one operand tile: the loader copies the whole tile, 8 rows (1 KiB) per
+// instruction.  Rows past the operand are clamped to its last row: what they bring in only reaches output
+// rows/columns that are never stored.  K must be a multiple of 64 (the host routes other shapes to the
+// generic kernels).
+template <int ROWS>
+struct DmaLane {
+  static constexpr int N = ROWS / 8;    // copies per K-step
+  const uint16_t* base;                 // uniform
+  uint32_t voff[N];                     // byte offset of this lane's granule from base at k0 = 0
+  __device__ __forceinline__ void init(const DmaOperand& op) {
+    const int lane = threadIdx.x & 63;
+    base = op.base;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int row = i * 8 + (lane >> 3);
+      const int kv = ((lane & 7) ^ ((row >> 1) & 7)) * 8;
+      const int r = min(row, op.rows - 1);
+      voff[i] = (uint32_t)(((size_t)r * op.ld + kv) * 2);
+    }
+  }
+  __device__ __forceinline__ void issue(int k0, uint32_t lds_tile) const {
+#pragma unroll
+    for (int i = 0; i < N; ++i) dma16(base + k0, voff[i], lds_tile + i * 1024);
+  }
+};
+
+__device__ __forceinline__ bf16x8 dma_fetch(const char* tile, int row, int kvec) {
+  const uint4 u = *reinterpret_cast<const uint4*>(tile + row * 128 + ((kvec ^ ((row >> 1) & 7)) << 4));
+  return __builtin_bit_cast(bf16x8, u);
+}
+
+template <class TS, int NBMAX, int STAGES>
+struct DmaSmem {
+  static constexpr int A_BYTES = TS::BM * 128, B_BYTES = TS::BN * 128;
+  static constexpr int STAGE = A_BYTES + NBMAX * B_BYTES;
+  static constexpr int BYTES = STAGE * STAGES;
+  static_assert(BYTES <= 160 * 1024, "ring does not fit the 160 KiB LDS");
+};
+
+constexpr int DMA_THREADS = 320;   // four MFMA waves + one loader wave
+
+// Flat multi-phase pipeline with a dedicated loader wave.
+//
+// A wave that issues a vector-memory instruction while the address FIFO is full stalls in order -- its
+// MFMAs stall with it -- and with four waves each copying a quarter of every tile the matrix pipe ran
+// dry for as long as the copies took (measured: K-step time = MFMA time + copy time).  So wave 4 issues
+// every copy (scalar bases, per-lane offsets precomputed: no vector ALU work per copy) and waves 0-3
+// only read fragments and issue MFMAs.  One barrier per K-step:
+//     loader:    wait until stage kt has landed; barrier; refill the stage the MFMA waves just left
+//     consumers: barrier; MFMAs on stage kt
+template <class TS, int NBMAX, int NPH, int STAGES>
+struct DmaPipe {
+  using SM = DmaSmem<TS, NBMAX, STAGES>;
+  static constexpr int loads(int nb) { return (TS::BM + nb * TS::BN) / 8; }   // loader copies per K-step
+
+  char* smem;
+  const DmaPhase<NBMAX>* ph;
+  int total;
+
+  __device__ __forceinline__ DmaPipe(char* s, const DmaPhase<NBMAX>* phases) : smem(s), ph(phases), total(0) {
+#pragma unroll
+    for (int i = 0; i < NPH; ++i) total += ph[i].K / DMA_BK;
+  }
+  __device__ static __forceinline__ bool is_loader() { return __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) == 4; }
+
+  // ---- loader wave: every copy of every phase.  MINLOADS: smallest per-K-step copy count of any phase.
+  template <int MINLOADS>
+  __device__ __forceinline__ void load_all() {
+    constexpr int AHEAD = (STAGES - 2) * MINLOADS > 63 ? 63 : (STAGES - 2) * MINLOADS;
+    DmaLane<TS::BM> la;
+    DmaLane<TS::BN> lb[NBMAX];
+    int cp = -1, ckt = 0, cnk = 0, cnb = 0, issued = 0;
+    auto next_phase = [&]() {
+      ++cp;
+      ckt = 0;
+#pragma unroll
+      for (int i = 0; i < NPH; ++i)
+        if (i == cp) {
+          la.init(ph[i].a);
+#pragma unroll
+          for (int j = 0; j < NBMAX; ++j) lb[j].init(ph[i].b[j]);
+          cnb = ph[i].nb;
+          cnk = ph[i].K / DMA_BK;
+        }
+    };
+    auto issue_stage = [&]() {
+      const uint32_t base = lds_addr(smem + (issued % STAGES) * SM::STAGE);
+      const int k0 = ckt * DMA_BK;
+      la.issue(k0, base);
+#pragma unroll
+      for (int j = 0; j < NBMAX; ++j)
+        if (j < cnb) lb[j].issue(k0, base + SM::A_BYTES + j * SM::B_BYTES);
+      ++issued;
+      if (++ckt == cnk && cp + 1 < NPH) next_phase();
+    };
+    next_phase();
+    for (int i = 0; i < STAGES - 1 && issued < total; ++i) issue_stage();
+    for (int kt = 0; kt < total; ++kt) {
+      if (kt + STAGES - 2 < total) wait_vmcnt<AHEAD>();
+      else wait_vmcnt<0>();
+      __syncthreads();
+      if (issued < total) issue_stage();
+    }
+  }
+
+  // ---- MFMA waves: one phase, nk K-steps into acc[0..NB).  `step` counts K-steps over all phases.
+  template <int NB>
+  __device__ __forceinline__ void run_phase(int nk, int& step, f32x16 (&acc)[NB][TS::TM][TS::TN]) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm0 = (wave / TS::WAVES_N) * TS::WM + (lane & 31), wn0 = (wave % TS::WAVES_N) * TS::WN + (lane & 31);
+    for (int kt = 0; kt < nk; ++kt, ++step) {
+      __syncthreads();
+      const char* st = smem + (step % STAGES) * SM::STAGE;
+      bf16x8 fa[2][TS::TM], fb[2][NB][TS::TN];
+      auto fetch = [&](int buf, int ks) {
+        const int kvec = ks * 2 + (lane >> 5);
+#pragma unroll
+        for (int i = 0; i < TS::TM; ++i) fa[buf][i] = dma_fetch(st, wm0 + i * 32, kvec);
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+#pragma unroll
+          for (int n = 0; n < TS::TN; ++n) fb[buf][j][n] = dma_fetch(st + SM::A_BYTES + j * SM::B_BYTES, wn0 + n * 32, kvec);
+      };
+      auto mfmas = [&](int buf) {
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+#pragma unroll
+          for (int i = 0; i < TS::TM; ++i)
+#pragma unroll
+            for (int n = 0; n < TS::TN; ++n) acc[j][i][n] = mma32(fb[buf][j][n], fa[buf][i], acc[j][i][n]);
+      };
+      fetch(0, 0);
+      fetch(1, 1);
+      mfmas(0);
+      fetch(0, 2);
+      mfmas(1);
+      fetch(1, 3);
+      mfmas(0);
+      mfmas(1);
+    }
+  }
+};
+
+// ---- epilogue staging: accumulators -> LDS tile -> whole rows ------------------------------------
+// A lane owns 4 consecutive n of 32 different rows per fragment; storing that straight to memory touches
+// 32 cache lines per instruction.  Staging the tile in LDS lets every store instruction cover whole rows.
+// Vector-ALU work bounds this phase, so all LDS addresses are (per-thread base + compile-time offset)
+// and the row loop advances pointers instead of dividing.
+//
+// StageTile<TS, E>: [BM][BN + PAD] elements of E bytes, 16-byte chunks; RPP rows are copied per pass.
+template <class TS, int E>
+struct StageTile {
+  static constexpr int CH = 16 / E;                    // elements per 16-byte chunk
+  static constexpr int LD = TS::BN + (E == 2 ? 8 : 4); // elements
+  static constexpr int BYTES = TS::BM * LD * E;
+  static constexpr int LPR = TS::BN / CH;              // lanes per row
+  static constexpr int RPP = TS::THREADS / LPR;        // rows per pass
+  static constexpr int PASSES = (TS::BM + RPP - 1) / RPP;
+
+  // byte offset inside the tile of this lane's first quad (fragment 0,0, g = 0)
+  __device__ static __forceinline__ int lane_base() {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int m = (wave / TS::WAVES_N) * TS::WM + (lane & 31), n = (wave % TS::WAVES_N) * TS::WN + 4 * (lane >> 5);
+    return (m * LD + n) * E;
+  }
+  // compile-time offset of fragment (tm, tn, g) relative to lane_base()
+  __device__ static constexpr int frag_off(int tm, int tn, int g) { return (tm * 32 * LD + tn * 32 + g * 8) * E; }
+  __device__ static __forceinline__ void put4(char* base, int tm, int tn, int g, float a, float b, float c, float d) {
+    if (E == 2) Elem<uint16_t>::store4(reinterpret_cast<uint16_t*>(base + frag_off(tm, tn, g)), a, b, c, d);
+    else *reinterpret_cast<float4*>(base + frag_off(tm, tn, g)) = make_float4(a, b, c, d);
+  }
+  // this thread's position in the copy-out phase
+  __device__ static __forceinline__ bool active() { return (int)threadIdx.x < RPP * LPR; }   // RPP*LPR <= 256: loader wave idle
+  __device__ static __forceinline__ int row0() { return threadIdx.x / LPR; }
+  __device__ static __forceinline__ int col0() { return (threadIdx.x % LPR) * CH; }
+};
+
+// Plain copy of a staged bf16 tile to `out` (row stride ld elements), rows/cols = valid extent of the tile.
+template <class TS>
+__device__ __forceinline__ void copy_out_b16(const char* smem, uint16_t* out, int ld, int rows, int cols) {
+  using ST = StageTile<TS, 2>;
+  if (!ST::active()) return;
+  const int r0 = ST::row0(), c0 = ST::col0();
+  if (c0 >= cols) return;
+  const char* src = smem + (r0 * ST::LD + c0) * 2;
+  uint16_t* dst = out + (size_t)r0 * ld + c0;
+  const size_t step = (size_t)ST::RPP * ld;
+#pragma unroll
+  for (int ps = 0; ps < ST::PASSES; ++ps) {
+    if (r0 + ps * ST::RPP < rows && r0 + ps * ST::RPP < TS::BM)
+      *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(src + ps * ST::RPP * ST::LD * 2);
+    dst += step;
+  }
+}
+
+}  // namespace lact

@@ -1,0 +1,440 @@
+// bf16 kernels of the TTT operation on the asynchronous-copy main loop (gemm_dma.h).
+// Same contractions and epilogues as gemm_kernels.h; all B operands K-contiguous (the host passes the
+// transposed bf16 copies of the small matrices where the contraction runs over their leading dimension).
+#pragma once
+#include "gemm_dma.h"
+#include "gemm_kernels.h"
+
+namespace lact {
+
+using TS_ROW = TileShape<256, 128, 2, 2>;   // token-row GEMMs, one accumulator: 128x64 per wave
+using TS_SQ = TileShape<128, 128, 2, 2>;    // small square GEMMs (Newton-Schulz) and 2-3 accumulator kernels
+using TS_BWD = TileShape<64, 128, 1, 4>;    // six accumulators (update backward): 64x32 per wave
+using TS_NS = TileShape<192, 192, 2, 2>;    // 384-multiple square GEMMs (Newton-Schulz at d = dh = 384): 96x96 per wave
+
+template <class TS> constexpr int row_stages() { return TS::BM == 128 ? 4 : 3; }
+
+// ------------------------------------------------------------------------------------------------
+// k_row_gemm_dma: out[M,N] = epilogue(sum_t A_t[M,K_t] * B_t[N,K_t]^T)
+// Extra outputs of the DUAL epilogue: out_ct = transposed copy in bf16 ([N][M] per matrix).
+// ------------------------------------------------------------------------------------------------
+template <int NT>
+struct RowGemmDmaParams {
+  RowGemmParams<NT> g;
+  uint16_t* out_ct;   // DUAL: bf16 transposed copy [N][M] (batch stride = bso), or null
+};
+
+template <class TS, int NT, int EPI>
+__global__ __launch_bounds__(DMA_THREADS) void k_row_gemm_dma(const RowGemmDmaParams<NT> pp) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr int STAGES = row_stages<TS>();
+  using Pipe = DmaPipe<TS, 1, NT, STAGES>;
+  const RowGemmParams<NT>& p = pp.g;
+  const int m0 = blockIdx.x * TS::BM, n0 = blockIdx.y * TS::BN, z = blockIdx.z;
+  DmaPhase<1> ph[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    ph[t].a.base = reinterpret_cast<const uint16_t*>(p.t[t].A) + z * p.t[t].bsA + (size_t)m0 * p.t[t].lda;
+    ph[t].a.ld = p.t[t].lda; ph[t].a.rows = p.M - m0;
+    ph[t].b[0].base = reinterpret_cast<const uint16_t*>(p.t[t].B) + z * p.t[t].bsB + (size_t)n0 * p.t[t].ldb;
+    ph[t].b[0].ld = p.t[t].ldb; ph[t].b[0].rows = p.N - n0;
+    ph[t].nb = 1;
+    ph[t].K = p.t[t].K;
+  }
+  f32x16 acc[1][TS::TM][TS::TN];
+  zero_acc<TS>(acc[0]);
+  LACT_TS(0);
+  Pipe pipe(smem, ph);
+  const bool loader = Pipe::is_loader();
+  LACT_TS(1);
+  if (loader) {
+    pipe.template load_all<Pipe::loads(1)>();
+  } else {
+    int step = 0;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) pipe.template run_phase<1>(p.t[t].K / DMA_BK, step, acc);
+  }
+  __syncthreads();
+  LACT_TS(2);
+
+  // ---- epilogue through an LDS-staged tile (see StageTile)
+  if (EPI != EPI_AXPBY_F32_DUAL) {
+    using ST = StageTile<TS, 2>;
+    char* lb = smem + ST::lane_base();
+    if (!loader) {
+      LACT_FOR_QUADS(TS) ST::put4(lb, tm, tn, g, acc[0][tm][tn][4 * g], acc[0][tm][tn][4 * g + 1], acc[0][tm][tn][4 * g + 2], acc[0][tm][tn][4 * g + 3]);
+    }
+    __syncthreads();
+    const int r0 = ST::row0(), c0 = ST::col0();
+    if (ST::active() && n0 + c0 < p.N) {
+      const char* src = smem + (r0 * ST::LD + c0) * 2;
+      uint16_t* dst = reinterpret_cast<uint16_t*>(p.out) + z * p.bso + (size_t)(m0 + r0) * p.ldo + n0 + c0;
+      const uint16_t* aux = reinterpret_cast<const uint16_t*>(p.aux) + z * p.bsaux + (size_t)(m0 + r0) * p.ldaux + n0 + c0;
+      const size_t dstep = (size_t)ST::RPP * p.ldo, astep = (size_t)ST::RPP * p.ldaux;
+      const bool blend = EPI == EPI_AXPBY || p.accumulate;
+      // all auxiliary loads first (no store in between may alias them), then blend and store
+      uint4 w[ST::PASSES];
+      if (blend) {
+        const uint16_t* ap = EPI == EPI_STORE ? dst : aux;
+        const size_t st = EPI == EPI_STORE ? dstep : astep;
+#pragma unroll
+        for (int ps = 0; ps < ST::PASSES; ++ps) {
+          const int r = r0 + ps * ST::RPP;
+          w[ps] = (r < TS::BM && m0 + r < p.M) ? *reinterpret_cast<const uint4*>(ap + ps * st) : make_uint4(0, 0, 0, 0);
+        }
+      }
+      const float al = EPI == EPI_STORE ? 1.f : p.alpha, be = EPI == EPI_STORE ? 1.f : p.beta;
+#pragma unroll
+      for (int ps = 0; ps < ST::PASSES; ++ps) {
+        const int r = r0 + ps * ST::RPP;
+        if (r < TS::BM && m0 + r < p.M) {
+          uint4 u = *reinterpret_cast<const uint4*>(src + ps * ST::RPP * ST::LD * 2);
+          if (blend) {
+            uint32_t uu[4] = {u.x, u.y, u.z, u.w}, ww[4] = {w[ps].x, w[ps].y, w[ps].z, w[ps].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const float lo = al * __uint_as_float(uu[j] << 16) + be * __uint_as_float(ww[j] << 16);
+              const float hi = al * __uint_as_float(uu[j] & 0xffff0000u) + be * __uint_as_float(ww[j] & 0xffff0000u);
+              uu[j] = (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+            }
+            u = make_uint4(uu[0], uu[1], uu[2], uu[3]);
+          }
+          *reinterpret_cast<uint4*>(dst) = u;
+        }
+        dst += dstep;
+      }
+    }
+  } else {
+    using ST = StageTile<TS, 4>;
+    char* lb = smem + ST::lane_base();
+    if (!loader) {
+      LACT_FOR_QUADS(TS) ST::put4(lb, tm, tn, g, acc[0][tm][tn][4 * g], acc[0][tm][tn][4 * g + 1], acc[0][tm][tn][4 * g + 2], acc[0][tm][tn][4 * g + 3]);
+    }
+    __syncthreads();
+    const bool tr = (p.transpose_mask >> (z / p.nb)) & 1;
+    const bool need_t = (p.out_t && tr) || pp.out_ct;
+    const int r0 = ST::row0(), c0 = ST::col0();
+    if (ST::active() && n0 + c0 < p.N) {
+      char* src = smem + (r0 * ST::LD + c0) * 4;
+      size_t off = z * p.bso + (size_t)(m0 + r0) * p.ldo + n0 + c0;
+      const float* aux = reinterpret_cast<const float*>(p.aux) + z * p.bsaux + (size_t)(m0 + r0) * p.ldaux + n0 + c0;
+      const size_t dstep = (size_t)ST::RPP * p.ldo, astep = (size_t)ST::RPP * p.ldaux;
+      float4 x4[ST::PASSES];
+#pragma unroll
+      for (int ps = 0; ps < ST::PASSES; ++ps) {
+        const int r = r0 + ps * ST::RPP;
+        x4[ps] = (r < TS::BM && m0 + r < p.M) ? *reinterpret_cast<const float4*>(aux + ps * astep) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int ps = 0; ps < ST::PASSES; ++ps) {
+        const int r = r0 + ps * ST::RPP;
+        if (r < TS::BM && m0 + r < p.M) {
+          float4* sp = reinterpret_cast<float4*>(src + ps * ST::RPP * ST::LD * 4);
+          const float4 a4 = *sp;
+          float v[4] = {p.alpha * a4.x + p.beta * x4[ps].x, p.alpha * a4.y + p.beta * x4[ps].y, p.alpha * a4.z + p.beta * x4[ps].z,
+                        p.alpha * a4.w + p.beta * x4[ps].w};
+          if (p.round_out_bf16) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = round_bf16(v[j]);
+          }
+          if (p.out) Elem<float>::store4(reinterpret_cast<float*>(p.out) + off, v[0], v[1], v[2], v[3]);
+          if (p.out_c) Elem<uint16_t>::store4(reinterpret_cast<uint16_t*>(p.out_c) + off, v[0], v[1], v[2], v[3]);
+          if (p.out_t && !tr) Elem<float>::store4(p.out_t + off, v[0], v[1], v[2], v[3]);
+          if (need_t) *sp = make_float4(v[0], v[1], v[2], v[3]);
+        }
+        off += dstep;
+      }
+    }
+    if (need_t) {
+      __syncthreads();
+      // transposed copies: lanes run along n (conflict-free LDS reads), each lane owns 8 consecutive m
+      const float* tile = reinterpret_cast<const float*>(smem);
+      constexpr int TP = TS::BN * (TS::BM / 8) / TS::THREADS;
+      static_assert(TS::THREADS % TS::BN == 0 || TS::BN % TS::THREADS == 0 || TS::BN == 192, "transposed pass mapping");
+#pragma unroll 2
+      for (int id = threadIdx.x; id < TS::BN * (TS::BM / 8); id += DMA_THREADS) {
+        const int nl = id % TS::BN, ml = (id / TS::BN) * 8;
+        const int m = m0 + ml, n = n0 + nl;
+        if (m >= p.M || n >= p.N) continue;
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = tile[(ml + j) * ST::LD + nl];
+        const size_t off = z * p.bso + (size_t)n * p.M + m;
+        if (p.out_t && tr) {
+          Elem<float>::store4(p.out_t + off, v[0], v[1], v[2], v[3]);
+          Elem<float>::store4(p.out_t + off + 4, v[4], v[5], v[6], v[7]);
+        }
+        if (pp.out_ct) {
+          Elem<uint16_t>::store4(pp.out_ct + off, v[0], v[1], v[2], v[3]);
+          Elem<uint16_t>::store4(pp.out_ct + off + 4, v[4], v[5], v[6], v[7]);
+        }
+      }
+      (void)TP;
+    }
+  }
+  LACT_TS(3);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Hidden-layer kernels.  W1T / G1T: transposed copies ([dh, d]) of w1 and of its gradient-of-gradient.
+// ------------------------------------------------------------------------------------------------
+struct HiddenDmaParams {
+  HiddenParams h;
+  const void* W1T; const void* G1T;
+};
+
+template <class TS>
+__device__ __forceinline__ DmaOperand token_operand(const void* base, long long bs, int ld, int z, int m0, int T) {
+  DmaOperand o;
+  o.base = reinterpret_cast<const uint16_t*>(base) + z * bs + (size_t)m0 * ld;
+  o.ld = ld;
+  o.rows = T - m0;
+  return o;
+}
+__device__ __forceinline__ DmaOperand weight_operand(const void* base, long long bs, int ld, int z, int n0, int rows) {
+  DmaOperand o;
+  o.base = reinterpret_cast<const uint16_t*>(base) + z * bs + (size_t)n0 * ld;
+  o.ld = ld;
+  o.rows = rows - n0;
+  return o;
+}
+
+// apply forward: O0 = silu(X W0^T) * (X W2^T)
+template <class TS>
+__global__ __launch_bounds__(DMA_THREADS) void k_apply_hidden_dma(const HiddenDmaParams pp) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr int STAGES = 3;
+  using Pipe = DmaPipe<TS, 2, 1, STAGES>;
+  const HiddenParams& p = pp.h;
+  const int m0 = blockIdx.x * TS::BM, n0 = blockIdx.y * TS::BN, z = blockIdx.z;
+  DmaPhase<2> ph[1];
+  ph[0].a = token_operand<TS>(p.X, p.bsx, p.ldx, z, m0, p.T);
+  ph[0].b[0] = weight_operand(p.W0, p.bsw, p.d, z, n0, p.dh);
+  ph[0].b[1] = weight_operand(p.W2, p.bsw, p.d, z, n0, p.dh);
+  ph[0].nb = 2;
+  ph[0].K = p.d;
+  const int nk = (p.d + DMA_BK - 1) / DMA_BK;
+  f32x16 acc[2][TS::TM][TS::TN];
+  zero_acc<TS>(acc[0]);
+  zero_acc<TS>(acc[1]);
+  LACT_TS(0);
+  Pipe pipe(smem, ph);
+  const bool loader = Pipe::is_loader();
+  LACT_TS(1);
+  if (loader) {
+    pipe.template load_all<Pipe::loads(2)>();
+  } else {
+    int step = 0;
+    pipe.template run_phase<2>(nk, step, acc);
+  }
+  __syncthreads();
+  LACT_TS(2);
+  using SB = StageTile<TS, 2>;
+  if (!loader) {
+    LACT_FOR_QUADS(TS) {
+      float v[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float y0 = round_bf16(acc[0][tm][tn][4 * g + j]), y2 = round_bf16(acc[1][tm][tn][4 * g + j]);
+        v[j] = round_bf16(y0 * sigmoidf_(y0)) * y2;
+      }
+      SB::put4(smem + SB::lane_base(), tm, tn, g, v[0], v[1], v[2], v[3]);
+    }
+  }
+  __syncthreads();
+  LACT_TS(3);
+  copy_out_b16<TS>(smem, reinterpret_cast<uint16_t*>(p.O0) + z * p.bso + (size_t)m0 * p.dh + n0, p.dh, p.T - m0, p.dh - n0);
+  LACT_TS(4);
+}
+
+// Shared main loop of the three-accumulator kernels: acc0 = X W0^T, acc1 = X W2^T, acc2 = Y W1 (via W1T).
+template <class TS>
+__device__ __forceinline__ void three_acc_mainloop(const HiddenDmaParams& pp, char* smem, int m0, int n0, int z,
+                                                   f32x16 (&a02)[2][TS::TM][TS::TN], f32x16 (&a1)[1][TS::TM][TS::TN]) {
+  constexpr int STAGES = 3;
+  using Pipe = DmaPipe<TS, 2, 2, STAGES>;
+  const HiddenParams& p = pp.h;
+  DmaPhase<2> ph[2];
+  ph[0].a = token_operand<TS>(p.X, p.bsx, p.ldx, z, m0, p.T);
+  ph[0].b[0] = weight_operand(p.W0, p.bsw, p.d, z, n0, p.dh);
+  ph[0].b[1] = weight_operand(p.W2, p.bsw, p.d, z, n0, p.dh);
+  ph[0].nb = 2;
+  ph[0].K = p.d;
+  ph[1].a = token_operand<TS>(p.Y, p.bsy, p.ldy, z, m0, p.T);
+  ph[1].b[0] = weight_operand(pp.W1T, p.bsw, p.d, z, n0, p.dh);
+  ph[1].b[1] = ph[1].b[0];
+  ph[1].nb = 1;
+  ph[1].K = p.d;
+  const int nk = (p.d + DMA_BK - 1) / DMA_BK;
+  zero_acc<TS>(a02[0]);
+  zero_acc<TS>(a02[1]);
+  zero_acc<TS>(a1[0]);
+  Pipe pipe(smem, ph);
+  if (Pipe::is_loader()) {
+    pipe.template load_all<Pipe::loads(1)>();
+  } else {
+    int step = 0;
+    pipe.template run_phase<2>(nk, step, a02);
+    pipe.template run_phase<1>(nk, step, a1);
+  }
+  __syncthreads();
+}
+
+template <class TS>
+__global__ __launch_bounds__(DMA_THREADS) void k_update_hidden_dma(const HiddenDmaParams pp) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const HiddenParams& p = pp.h;
+  const int m0 = blockIdx.x * TS::BM, n0 = blockIdx.y * TS::BN, z = blockIdx.z;
+  f32x16 a02[2][TS::TM][TS::TN], a1[1][TS::TM][TS::TN];
+  three_acc_mainloop<TS>(pp, smem, m0, n0, z, a02, a1);
+  using SB = StageTile<TS, 2>;
+  char* s0 = smem + SB::lane_base(); char* s1 = s0 + SB::BYTES; char* s2 = s0 + 2 * SB::BYTES;
+  const int ntm = threadIdx.x < TS::THREADS ? TS::TM : 0;   // the loader wave owns no fragments
+#pragma unroll
+  for (int tm = 0; tm < TS::TM; ++tm) {
+    if (tm >= ntm) break;
+    const int ml = quad_m<TS>(tm), m = m0 + ml;
+    const bool mv = m < p.T;
+    const float l0 = mv ? p.lr0[z * p.bslr + m] : 0.f, l1 = mv ? p.lr1[z * p.bslr + m] : 0.f;
+    const float l2 = mv ? p.lr2[z * p.bslr + m] : 0.f;
+#pragma unroll
+    for (int tn = 0; tn < TS::TN; ++tn)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        float z0[4], z1[4], z2[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float gg = round_bf16(a02[0][tm][tn][4 * g + j]), h2 = round_bf16(a02[1][tm][tn][4 * g + j]);
+          const float dh = round_bf16(a1[0][tm][tn][4 * g + j]);
+          const UpdatePointwise u = update_pointwise<uint16_t>(gg, h2, dh, silu_parts(gg));
+          z0[j] = u.dgpre * l0; z1[j] = u.hid * l1; z2[j] = u.dh2 * l2;
+        }
+        SB::put4(s0, tm, tn, g, z0[0], z0[1], z0[2], z0[3]);
+        SB::put4(s1, tm, tn, g, z1[0], z1[1], z1[2], z1[3]);
+        SB::put4(s2, tm, tn, g, z2[0], z2[1], z2[2], z2[3]);
+      }
+  }
+  __syncthreads();
+  const size_t off = z * p.bso + (size_t)m0 * p.dh + n0;
+  copy_out_b16<TS>(smem + 0 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O0) + off, p.dh, p.T - m0, p.dh - n0);
+  copy_out_b16<TS>(smem + 1 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O1) + off, p.dh, p.T - m0, p.dh - n0);
+  copy_out_b16<TS>(smem + 2 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O2) + off, p.dh, p.T - m0, p.dh - n0);
+}
+
+template <class TS>
+__global__ __launch_bounds__(DMA_THREADS) void k_apply_bwd_hidden_dma(const HiddenDmaParams pp) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const HiddenParams& p = pp.h;
+  const int m0 = blockIdx.x * TS::BM, n0 = blockIdx.y * TS::BN, z = blockIdx.z;
+  f32x16 a02[2][TS::TM][TS::TN], a1[1][TS::TM][TS::TN];
+  three_acc_mainloop<TS>(pp, smem, m0, n0, z, a02, a1);
+  using SB = StageTile<TS, 2>;
+  char* s0 = smem + SB::lane_base(); char* s1 = s0 + SB::BYTES; char* s2 = s0 + 2 * SB::BYTES;
+  if (threadIdx.x < TS::THREADS) LACT_FOR_QUADS(TS) {
+    float hq[4], gy0[4], gy2[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float y0 = round_bf16(a02[0][tm][tn][4 * g + j]), y2 = round_bf16(a02[1][tm][tn][4 * g + j]);
+      const float gh = round_bf16(a1[0][tm][tn][4 * g + j]);
+      const SiluParts s = silu_parts(y0);
+      const float sg = round_bf16(s.silu);
+      hq[j] = sg * y2; gy0[j] = gh * y2 * s.d1; gy2[j] = gh * sg;
+    }
+    SB::put4(s0, tm, tn, g, hq[0], hq[1], hq[2], hq[3]);
+    SB::put4(s1, tm, tn, g, gy0[0], gy0[1], gy0[2], gy0[3]);
+    SB::put4(s2, tm, tn, g, gy2[0], gy2[1], gy2[2], gy2[3]);
+  }
+  __syncthreads();
+  const size_t off = z * p.bso + (size_t)m0 * p.dh + n0;
+  copy_out_b16<TS>(smem + 0 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O0) + off, p.dh, p.T - m0, p.dh - n0);
+  copy_out_b16<TS>(smem + 1 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O1) + off, p.dh, p.T - m0, p.dh - n0);
+  copy_out_b16<TS>(smem + 2 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O2) + off, p.dh, p.T - m0, p.dh - n0);
+}
+
+// update backward, hidden stage: phases (X; W0,W2), (X; G0,G2), (Y; W1T,G1T)
+template <class TS>
+__global__ __launch_bounds__(DMA_THREADS) void k_update_bwd_hidden_dma(const HiddenDmaParams pp) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr int STAGES = 3;
+  using Pipe = DmaPipe<TS, 2, 3, STAGES>;
+  const HiddenParams& p = pp.h;
+  const int m0 = blockIdx.x * TS::BM, n0 = blockIdx.y * TS::BN, z = blockIdx.z;
+  DmaPhase<2> ph[3];
+  ph[0].a = token_operand<TS>(p.X, p.bsx, p.ldx, z, m0, p.T);
+  ph[0].b[0] = weight_operand(p.W0, p.bsw, p.d, z, n0, p.dh);
+  ph[0].b[1] = weight_operand(p.W2, p.bsw, p.d, z, n0, p.dh);
+  ph[1].a = ph[0].a;
+  ph[1].b[0] = weight_operand(p.G0, p.bsw, p.d, z, n0, p.dh);
+  ph[1].b[1] = weight_operand(p.G2, p.bsw, p.d, z, n0, p.dh);
+  ph[2].a = token_operand<TS>(p.Y, p.bsy, p.ldy, z, m0, p.T);
+  ph[2].b[0] = weight_operand(pp.W1T, p.bsw, p.d, z, n0, p.dh);
+  ph[2].b[1] = weight_operand(pp.G1T, p.bsw, p.d, z, n0, p.dh);
+  ph[0].K = ph[1].K = ph[2].K = p.d;
+  ph[0].nb = ph[1].nb = ph[2].nb = 2;
+  const int nk = (p.d + DMA_BK - 1) / DMA_BK;
+  f32x16 aw[2][TS::TM][TS::TN], ag[2][TS::TM][TS::TN], ay[2][TS::TM][TS::TN];
+  zero_acc<TS>(aw[0]); zero_acc<TS>(aw[1]); zero_acc<TS>(ag[0]); zero_acc<TS>(ag[1]); zero_acc<TS>(ay[0]); zero_acc<TS>(ay[1]);
+  Pipe pipe(smem, ph);
+  const bool loader = Pipe::is_loader();
+  if (loader) {
+    pipe.template load_all<Pipe::loads(2)>();
+  } else {
+    int step = 0;
+    pipe.template run_phase<2>(nk, step, aw);
+    pipe.template run_phase<2>(nk, step, ag);
+    pipe.template run_phase<2>(nk, step, ay);
+  }
+  __syncthreads();
+  using SB = StageTile<TS, 2>;
+  char* lb = smem + SB::lane_base();
+  if (!loader) {
+#pragma unroll
+  for (int tm = 0; tm < TS::TM; ++tm) {
+    const int ml = quad_m<TS>(tm), m = m0 + ml;
+    const bool mv = m < p.T;
+    const float l0 = mv ? p.lr0[z * p.bslr + m] : 0.f, l1 = mv ? p.lr1[z * p.bslr + m] : 0.f;
+    const float l2 = mv ? p.lr2[z * p.bslr + m] : 0.f;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int tn = 0; tn < TS::TN; ++tn)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int nl = quad_n<TS>(tn, g);
+        const bool nv = n0 + nl < p.dh;
+        float o0[4], o1[4], o2[4], o3[4], o4[4], o5[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float gg = round_bf16(aw[0][tm][tn][4 * g + j]), h2 = round_bf16(aw[1][tm][tn][4 * g + j]);
+          const float dh = round_bf16(ay[0][tm][tn][4 * g + j]);
+          const float gz0 = round_bf16(ag[0][tm][tn][4 * g + j]), gz2 = round_bf16(ag[1][tm][tn][4 * g + j]);
+          const float gz1 = round_bf16(ay[1][tm][tn][4 * g + j]);
+          const SiluParts s = silu_parts(gg);
+          const UpdatePointwise u = update_pointwise<uint16_t>(gg, h2, dh, s);
+          if (mv && nv) { s0 += gz0 * u.dgpre; s1 += gz1 * u.hid; s2 += gz2 * u.dh2; }
+          const float ghid = gz1 * l1, gdh2 = gz2 * l2, gdg = gz0 * l0;
+          o0[j] = ghid * h2 * s.d1 + gdh2 * dh * s.d1 + gdg * dh * h2 * s.d2;
+          o1[j] = gdh2 * s.silu + gdg * h2 * s.d1;
+          o2[j] = ghid * s.silu + gdg * dh * s.d1;
+          o3[j] = u.dgpre * l0; o4[j] = u.hid * l1; o5[j] = u.dh2 * l2;
+        }
+        SB::put4(lb + 0 * SB::BYTES, tm, tn, g, o0[0], o0[1], o0[2], o0[3]);
+        SB::put4(lb + 1 * SB::BYTES, tm, tn, g, o1[0], o1[1], o1[2], o1[3]);
+        SB::put4(lb + 2 * SB::BYTES, tm, tn, g, o2[0], o2[1], o2[2], o2[3]);
+        SB::put4(lb + 3 * SB::BYTES, tm, tn, g, o3[0], o3[1], o3[2], o3[3]);
+        SB::put4(lb + 4 * SB::BYTES, tm, tn, g, o4[0], o4[1], o4[2], o4[3]);
+        SB::put4(lb + 5 * SB::BYTES, tm, tn, g, o5[0], o5[1], o5[2], o5[3]);
+      }
+    store_row_partials<TS>(p, 0, tm, m, z, s0);
+    store_row_partials<TS>(p, 1, tm, m, z, s1);
+    store_row_partials<TS>(p, 2, tm, m, z, s2);
+  }
+  }
+  __syncthreads();
+  const size_t off = z * p.bso + (size_t)m0 * p.dh + n0;
+  void* outs[6] = {p.O0, p.O1, p.O2, p.O3, p.O4, p.O5};
+#pragma unroll
+  for (int i = 0; i < 6; ++i)
+    copy_out_b16<TS>(smem + i * SB::BYTES, reinterpret_cast<uint16_t*>(outs[i]) + off, p.dh, p.T - m0, p.dh - n0);
+}
+
+}  // namespace lact

@@ -9,6 +9,9 @@
 #include <string>
 #include <vector>
 
+#include <type_traits>
+
+#include "gemm_dma_kernels.h"
 #include "gemm_kernels.h"
 #include "state_kernels.h"
 
@@ -72,6 +75,18 @@ struct ProfScope {
     hipLaunchKernelGGL(kern, grid, block, 0, stream, __VA_ARGS__);      \
   } while (0)
 
+#define LACT_LAUNCH_SMEM(kname, site, flops, kern, grid, block, smem_bytes, stream, ...) \
+  do {                                                                                   \
+    ProfScope ps_(kname, site, flops, stream);                                           \
+    hipLaunchKernelGGL(kern, grid, block, smem_bytes, stream, __VA_ARGS__);              \
+  } while (0)
+
+// kernels whose ring exceeds the default dynamic LDS limit opt in once per instantiation
+template <class K>
+void allow_big_lds(K kern, int bytes) {
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+}
+
 template <typename T> const char* tname();
 template <> const char* tname<uint16_t>() { return "bf16"; }
 template <> const char* tname<float>() { return "f32"; }
@@ -115,10 +130,10 @@ struct Plan {
   bool muon = false, bf16 = true, momentum = false;
   size_t mat3 = 0;  // 3*b*elems
   // saved
-  size_t s_n0, s_wf, s_wc, s_main, s_d, s_mbar, s_u, s_g16, s_norms, s_xb, s_ab, s_bb, saved_bytes;
+  size_t s_wct, s_xbt, s_n0, s_wf, s_wc, s_main, s_d, s_mbar, s_u, s_g16, s_norms, s_xb, s_ab, s_bb, saved_bytes;
   // scratch
   size_t t_h[6], t_partial, t_lrpart, t_xf[2], t_xbtmp, t_ss, t_dot, t_mdot, t_gwhat[2], t_gwcur, t_gmcarry, t_gc,
-      t_gxf[2], t_gxb[2], t_sg, t_gas, t_gn0, scratch_bytes;
+      t_gxf[2], t_gxb[2], t_sg, t_gas, t_gn0, t_gct, t_gxbt[2], scratch_bytes;
 
   int build(const lact_desc_t* desc) {
     if (!desc) return fail("null descriptor");
@@ -166,7 +181,7 @@ struct Plan {
     c = std::max(d.d, d.dh);
     mat3 = (size_t)3 * d.b * g.elems;
     nblk = std::max(1, std::min(256, (int)((g.elems + 2047) / 2048)));
-    lr_slots = ceil_div(d.dh, TSB::BN) * TSB::WAVES_N;
+    lr_slots = ceil_div(d.dh, 128) * 4;   // (hidden tiles) x (wave columns) of the widest update-backward tiling
     tiles = ceil_div(d.dh, TSA::BM) * ceil_div(d.d, TSA::BN);
     tiles = std::max(tiles, ceil_div(d.d, TSA::BM) * ceil_div(d.dh, TSA::BN));
     nsplit_max = choose_split(Tcap, tiles * 3 * d.b).n;
@@ -175,6 +190,7 @@ struct Plan {
     s_n0 = sv.take((size_t)3 * d.b * g.maxrows() * 4);
     s_wf = sv.take((size_t)(nupd + 1) * mat3 * 4);
     s_wc = bf16 ? sv.take((size_t)(nupd + 1) * mat3 * 2) : s_wf;
+    s_wct = bf16 ? sv.take((size_t)(nupd + 1) * mat3 * 2) : 0;
     s_main = d.prenorm ? sv.take((size_t)nupd * mat3 * 4) : 0;
     s_d = sv.take((size_t)nupd * mat3 * 4);
     s_mbar = sv.take((size_t)std::max(1, nupd) * d.b * 4);
@@ -182,6 +198,7 @@ struct Plan {
     s_g16 = muon ? sv.take((size_t)nupd * mat3 * nsz) : 0;
     s_norms = sv.take((size_t)std::max(1, nupd) * 3 * d.b * 4);
     s_xb = muon ? sv.take((size_t)nupd * std::max(1, S) * mat3 * nsz) : 0;
+    s_xbt = (muon && nsz == 2) ? sv.take((size_t)nupd * std::max(1, S) * mat3 * 2) : 0;
     const size_t sq3 = (size_t)3 * d.b * r * r;
     s_ab = muon ? sv.take((size_t)nupd * std::max(1, S) * sq3 * nsz) : 0;
     s_bb = muon ? sv.take((size_t)nupd * std::max(1, S) * sq3 * nsz) : 0;
@@ -205,6 +222,8 @@ struct Plan {
     t_sg = sc.take(sq3 * nsz);
     t_gas = sc.take(sq3 * nsz);
     t_gn0 = sc.take((size_t)3 * d.b * g.maxrows() * 4);
+    t_gct = sc.take(mat3 * 2);
+    for (int i = 0; i < 2; ++i) t_gxbt[i] = sc.take(mat3 * 2);
     scratch_bytes = sc.off + 256;
     return 0;
   }
@@ -221,8 +240,46 @@ const char* row_gemm_name() {
                                (EPI == EPI_STORE ? ",store>" : (EPI == EPI_AXPBY ? ",axpby>" : ",axpby_dual>"));
   return n.c_str();
 }
+// transposed ([N][K], K contiguous) copy of a K-strided B operand, for the asynchronous-copy kernels
+struct BT {
+  const void* p;
+  int ld;
+};
+template <class TS, int NT, int EPI>
+void launch_row_gemm_dma(const char* site, const RowGemmDmaParams<NT>& q, int batch, hipStream_t s) {
+  constexpr int STAGES = row_stages<TS>();
+  constexpr int SMEM = cmax(DmaSmem<TS, 1, STAGES>::BYTES, StageTile<TS, 4>::BYTES);
+  static bool once = (allow_big_lds(k_row_gemm_dma<TS, NT, EPI>, SMEM), true);
+  (void)once;
+  static const std::string name = std::string("k_row_gemm_dma<") + std::to_string(TS::BM) + "x" + std::to_string(TS::BN) + "," +
+                                  std::to_string(NT) + (EPI == EPI_STORE ? ",store>" : (EPI == EPI_AXPBY ? ",axpby>" : ",axpby_dual>"));
+  dim3 grid(ceil_div(q.g.M, TS::BM), ceil_div(q.g.N, TS::BN), batch);
+  double ksum = 0;
+  for (int t = 0; t < NT; ++t) ksum += q.g.t[t].K;
+  LACT_LAUNCH_SMEM(name.c_str(), site, 2.0 * q.g.M * q.g.N * ksum * batch, (k_row_gemm_dma<TS, NT, EPI>), grid, dim3(DMA_THREADS),
+                   SMEM, s, q);
+}
 template <typename T, bool B_KC, int NT, int EPI>
-void launch_row_gemm(const char* site, const RowGemmParams<NT>& p, int batch, hipStream_t s) {
+void launch_row_gemm(const char* site, const RowGemmParams<NT>& p, int batch, hipStream_t s, const BT* bt = nullptr,
+                     uint16_t* out_ct = nullptr, bool token_rows = false) {
+  if constexpr (std::is_same<T, uint16_t>::value) {
+    bool k64 = true;
+    for (int t = 0; t < NT; ++t) k64 = k64 && p.t[t].K % 64 == 0;
+    if ((B_KC || bt) && k64) {
+      RowGemmDmaParams<NT> q;
+      q.g = p;
+      q.out_ct = out_ct;
+      if (!B_KC)
+        for (int t = 0; t < NT; ++t) {
+          q.g.t[t].B = bt[t].p;
+          q.g.t[t].ldb = bt[t].ld;
+        }
+      if (token_rows) launch_row_gemm_dma<TS_ROW, NT, EPI>(site, q, batch, s);
+      else if (p.M % TS_NS::BM == 0 && p.N % TS_NS::BN == 0) launch_row_gemm_dma<TS_NS, NT, EPI>(site, q, batch, s);
+      else launch_row_gemm_dma<TS_SQ, NT, EPI>(site, q, batch, s);
+      return;
+    }
+  }
   dim3 grid(ceil_div(p.M, TSA::BM), ceil_div(p.N, TSA::BN), batch);
   double ksum = 0;
   for (int t = 0; t < NT; ++t) ksum += p.t[t].K;
@@ -253,6 +310,7 @@ struct NsIter {
   const float* xf_in; const void* xb_in;           // X: fp32 iterate and its copy in the GEMM type
   void* ab; void* bb;                              // A and B of this iteration (GEMM type)
   float* xf_out; void* xb_out; float* u_out;       // X': fp32, GEMM type, and fp32 in the original orientation (each nullable)
+  const uint16_t* xbt_in; uint16_t* xbt_out;       // bf16 [c][r] copies of X and X' (asynchronous-copy kernels), nullable
 };
 // TN: GEMM operand type of the iteration (bf16 as in the reference, or fp32 for the exact mode)
 template <typename TN>
@@ -279,7 +337,8 @@ void ns_iteration(const NsIter& I, hipStream_t s) {
     p.round_out_bf16 = I.plain;
     p.out = I.xf_out; p.out_c = I.xb_out; p.out_t = I.u_out;
     p.transpose_mask = I.mask; p.nb = I.nb_for_mask;
-    launch_row_gemm<TN, false, 1, EPI_AXPBY_F32_DUAL>("ns_next", p, I.n, s);
+    const BT bt[1] = {{I.xbt_in, I.r}};
+    launch_row_gemm<TN, false, 1, EPI_AXPBY_F32_DUAL>("ns_next", p, I.n, s, I.xbt_in ? bt : nullptr, I.xbt_out);
   }
 }
 
@@ -309,6 +368,60 @@ struct Runner {
   TN* ab(int u, int it) const { return reinterpret_cast<TN*>(sv + P.s_ab) + ((size_t)u * std::max(1, P.S) + it) * sq3(); }
   TN* bb(int u, int it) const { return reinterpret_cast<TN*>(sv + P.s_bb) + ((size_t)u * std::max(1, P.S) + it) * sq3(); }
   T* h(int i) const { return reinterpret_cast<T*>(sc + P.t_h[i]); }
+  // bf16 activations: transposed bf16 copies of the small matrices feed the asynchronous-copy kernels
+  static constexpr bool kBf16 = std::is_same<T, uint16_t>::value;
+  static constexpr bool kNsBf16 = std::is_same<TN, uint16_t>::value;
+  uint16_t* wct(int ver) const { return kBf16 ? reinterpret_cast<uint16_t*>(sv + P.s_wct) + (size_t)ver * P.mat3 : nullptr; }
+  uint16_t* wct(int ver, int j) const { return kBf16 ? wct(ver) + (size_t)j * d.b * P.g.elems : nullptr; }
+  uint16_t* xbt(int u, int it) const {
+    return kNsBf16 ? reinterpret_cast<uint16_t*>(sv + P.s_xbt) + ((size_t)u * std::max(1, P.S) + it) * P.mat3 : nullptr;
+  }
+  uint16_t* gct() const { return kBf16 ? reinterpret_cast<uint16_t*>(sc + P.t_gct) : nullptr; }
+  uint16_t* gct(int j) const { return kBf16 ? gct() + (size_t)j * d.b * P.g.elems : nullptr; }
+  uint16_t* gxbt(int i) const { return kNsBf16 ? reinterpret_cast<uint16_t*>(sc + P.t_gxbt[i]) : nullptr; }
+
+  // bf16 transposed copies of packed small matrices (weight orientation or Newton-Schulz orientation)
+  void transpose3(const void* src, uint16_t* dst, bool ns_orientation) const {
+    if (!dst) return;
+    TransposeParams p;
+    p.src = reinterpret_cast<const uint16_t*>(src); p.dst = dst; p.nb = d.b; p.elems = P.g.elems;
+    int mr = 0, mc = 0;
+    for (int j = 0; j < 3; ++j) {
+      p.rows[j] = ns_orientation ? P.r : P.g.rows(j);
+      p.cols[j] = ns_orientation ? P.c : P.g.cols(j);
+      mr = std::max(mr, p.rows[j]); mc = std::max(mc, p.cols[j]);
+    }
+    LACT_LAUNCH("k_transpose_b16", "k_transpose_b16", 0.0, k_transpose_b16, dim3(ceil_div(mc, 64), ceil_div(mr, 64), 3 * d.b), dim3(256), s, p);
+  }
+
+  // the four hidden-layer kernels: asynchronous-copy version for bf16, generic tile loop otherwise
+  void launch_hidden(int which, const HiddenParams& hp, int ver, const uint16_t* g1t, int T_) const {
+    const double f = (double)T_ * d.d * d.dh * d.b;
+    if (kBf16 && d.d % 64 == 0) {
+      if constexpr (kBf16) {
+      HiddenDmaParams q;
+      q.h = hp;
+      q.W1T = wct(ver, 1);
+      q.G1T = g1t;
+      constexpr int SM3 = cmax(DmaSmem<TS_SQ, 2, 3>::BYTES, 3 * StageTile<TS_SQ, 2>::BYTES);
+      constexpr int SM6 = cmax(DmaSmem<TS_BWD, 2, 3>::BYTES, 6 * StageTile<TS_BWD, 2>::BYTES);
+      dim3 g3(ceil_div(T_, TS_SQ::BM), ceil_div(d.dh, TS_SQ::BN), d.b), g6(ceil_div(T_, TS_BWD::BM), ceil_div(d.dh, TS_BWD::BN), d.b);
+      static bool once = (allow_big_lds(k_apply_hidden_dma<TS_SQ>, SM3), allow_big_lds(k_update_hidden_dma<TS_SQ>, SM3),
+                          allow_big_lds(k_apply_bwd_hidden_dma<TS_SQ>, SM3), allow_big_lds(k_update_bwd_hidden_dma<TS_BWD>, SM6), true);
+      (void)once;
+      if (which == 0) LACT_LAUNCH_SMEM("k_apply_hidden_dma", "apply_hidden", 4.0 * f, (k_apply_hidden_dma<TS_SQ>), g3, dim3(DMA_THREADS), SM3, s, q);
+      if (which == 1) LACT_LAUNCH_SMEM("k_update_hidden_dma", "update_hidden", 6.0 * f, (k_update_hidden_dma<TS_SQ>), g3, dim3(DMA_THREADS), SM3, s, q);
+      if (which == 2) LACT_LAUNCH_SMEM("k_apply_bwd_hidden_dma", "apply_bwd_hidden", 6.0 * f, (k_apply_bwd_hidden_dma<TS_SQ>), g3, dim3(DMA_THREADS), SM3, s, q);
+      if (which == 3) LACT_LAUNCH_SMEM("k_update_bwd_hidden_dma", "update_bwd_hidden", 12.0 * f, (k_update_bwd_hidden_dma<TS_BWD>), g6, dim3(DMA_THREADS), SM6, s, q);
+      }
+    } else {
+      dim3 ga(ceil_div(T_, TSA::BM), ceil_div(d.dh, TSA::BN), d.b), gb(ceil_div(T_, TSB::BM), ceil_div(d.dh, TSB::BN), d.b);
+      if (which == 0) LACT_LAUNCH("k_apply_hidden", "apply_hidden", 4.0 * f, (k_apply_hidden<T, TSA>), ga, dim3(TSA::THREADS), s, hp);
+      if (which == 1) LACT_LAUNCH("k_update_hidden", "update_hidden", 6.0 * f, (k_update_hidden<T, TSA>), ga, dim3(TSA::THREADS), s, hp);
+      if (which == 2) LACT_LAUNCH("k_apply_bwd_hidden", "apply_bwd_hidden", 6.0 * f, (k_apply_bwd_hidden<T, TSA>), ga, dim3(TSA::THREADS), s, hp);
+      if (which == 3) LACT_LAUNCH("k_update_bwd_hidden", "update_bwd_hidden", 12.0 * f, (k_update_bwd_hidden<T, TSB>), gb, dim3(TSB::THREADS), s, hp);
+    }
+  }
   template <typename U> U* scr(size_t off) const { return reinterpret_cast<U*>(sc + off); }
 
   int tall_mask() const { return (P.g.tall(0) ? 1 : 0) | (P.g.tall(1) ? 2 : 0) | (P.g.tall(2) ? 4 : 0); }
@@ -359,7 +472,9 @@ struct Runner {
       InitParams p;
       p.g = P.g; p.w[0] = w0; p.w[1] = w1; p.w[2] = w2; p.n0 = n0(); p.wf = wf(0);
       p.wc = P.bf16 ? (void*)wc(0) : nullptr;
+      p.wct = nullptr;
       LACT_LAUNCH("k_init_state", "k_init_state", 0.0, (k_init_state<T>), rowgrid, dim3(256), s, p);
+      if (kBf16) transpose3(wc(0), wct(0), false);
     }
     int ver = 0, u = 0;
     for (const auto& st : P.steps) {
@@ -367,12 +482,11 @@ struct Runner {
       if (st.kind == LACT_APPLY) {
         HiddenParams hp = hidden_params(T_, q + (size_t)st.start * d.q_ld, d.q_ld, d.q_bs, nullptr, 0, 0, ver);
         hp.O0 = h(0);
-        dim3 grid(ceil_div(T_, TSA::BM), ceil_div(d.dh, TSA::BN), d.b);
-        LACT_LAUNCH("k_apply_hidden", "apply_hidden", 4.0 * T_ * d.d * d.dh * d.b, (k_apply_hidden<T, TSA>), grid, dim3(TSA::THREADS), s, hp);
+        launch_hidden(0, hp, ver, nullptr, T_);
         auto p = row_params<1>();
         set_term(p.t[0], h(0), d.dh, hbs(), wc(ver, 1), d.dh, P.g.elems, d.dh);
         p.M = T_; p.N = d.d; p.out = out + (size_t)st.out_start * d.o_ld; p.ldo = d.o_ld; p.bso = d.o_bs;
-        launch_row_gemm<T, true, 1, EPI_STORE>("apply_out", p, d.b, s);
+        launch_row_gemm<T, true, 1, EPI_STORE>("apply_out", p, d.b, s, nullptr, nullptr, true);
         continue;
       }
       // ---- update
@@ -382,8 +496,7 @@ struct Runner {
         HiddenParams hp = hidden_params(T_, kc, d.k_ld, d.k_bs, vc, d.v_ld, d.v_bs, ver);
         hp.lr0 = lr0 + st.start; hp.lr1 = lr1 + st.start; hp.lr2 = lr2 + st.start; hp.bslr = d.kv_len;
         hp.O0 = h(0); hp.O1 = h(1); hp.O2 = h(2);
-        dim3 grid(ceil_div(T_, TSA::BM), ceil_div(d.dh, TSA::BN), d.b);
-        LACT_LAUNCH("k_update_hidden", "update_hidden", 6.0 * T_ * d.d * d.dh * d.b, (k_update_hidden<T, TSA>), grid, dim3(TSA::THREADS), s, hp);
+        launch_hidden(1, hp, ver, nullptr, T_);
       }
       const Split sp = choose_split(T_, P.tiles * 3 * d.b);
       {
@@ -416,9 +529,11 @@ struct Runner {
         memset(&p, 0, sizeof(p));
         p.g = P.g; p.g16 = g16(u); p.ss_part = scr<float>(P.t_ss); p.nparts = P.nblk; p.norms = norms(u);
         p.xf = scr<float>(P.t_xf[0]); p.xb = xb(u, 0);
+        p.xbt = nullptr;
         p.u = P.S == 0 ? usave(u) : nullptr;
         p.plain_bf16 = d.ns_mode == LACT_NS_PLAIN_BF16;
         LACT_LAUNCH("k_ns_scale", "k_ns_scale", 0.0, (k_ns_scale<TN>), dim3(P.nblk, 3 * d.b), dim3(256), s, p);
+        if (kNsBf16 && P.S > 0) transpose3(xb(u, 0), xbt(u, 0), true);
         for (int it = 0; it < P.S; ++it) {
           const bool last = it + 1 == P.S;
           NsIter I;
@@ -429,6 +544,7 @@ struct Runner {
           I.xf_out = last ? nullptr : scr<float>(P.t_xf[(it + 1) & 1]);
           I.xb_out = last ? (void*)scr<TN>(P.t_xbtmp) : (void*)xb(u, it + 1);
           I.u_out = last ? usave(u) : nullptr;
+          I.xbt_in = xbt(u, it); I.xbt_out = last ? nullptr : xbt(u, it + 1);
           ns_iteration<TN>(I, s);
         }
       }
@@ -437,7 +553,9 @@ struct Runner {
         p.main_out = d.prenorm ? main_(u + 1) : nullptr;
         p.wf_out = wf(ver + 1);
         p.wc_out = P.bf16 ? (void*)wc(ver + 1) : nullptr;
+        p.wct_out = nullptr;
         LACT_LAUNCH("k_update_renorm", "k_update_renorm", 0.0, (k_update_renorm<T>), rowgrid, dim3(256), s, p);
+        if (kBf16) transpose3(wc(ver + 1), wct(ver + 1), false);
       }
       ++ver;
       ++u;
@@ -492,15 +610,15 @@ struct Runner {
         const T* gc = dout + (size_t)st.out_start * d.do_ld;
         HiddenParams hp = hidden_params(T_, qc, d.q_ld, d.q_bs, gc, d.do_ld, d.do_bs, ver);
         hp.O0 = h(0); hp.O1 = h(1); hp.O2 = h(2);
-        dim3 grid(ceil_div(T_, TSA::BM), ceil_div(d.dh, TSA::BN), d.b);
-        LACT_LAUNCH("k_apply_bwd_hidden", "apply_bwd_hidden", 6.0 * T_ * d.d * d.dh * d.b, (k_apply_bwd_hidden<T, TSA>), grid, dim3(TSA::THREADS), s, hp);
+        launch_hidden(2, hp, ver, nullptr, T_);
         {  // dq = gY0 W0 + gY2 W2
           auto p = row_params<2>();
           set_term(p.t[0], h(1), d.dh, hbs(), wc(ver, 0), d.d, P.g.elems, d.dh);
           set_term(p.t[1], h(2), d.dh, hbs(), wc(ver, 2), d.d, P.g.elems, d.dh);
           p.M = T_; p.N = d.d; p.out = dq + (size_t)st.start * d.d; p.ldo = d.d; p.bso = (long long)d.q_len * d.d;
           p.accumulate = overlaps(seen_q, st.start, st.end);
-          launch_row_gemm<T, false, 2, EPI_STORE>("apply_bwd_dq", p, d.b, s);
+          const BT bt[2] = {{wct(ver, 0), d.dh}, {wct(ver, 2), d.dh}};
+          launch_row_gemm<T, false, 2, EPI_STORE>("apply_bwd_dq", p, d.b, s, kBf16 ? bt : nullptr, nullptr, true);
         }
         TokenReduceJob jobs[3];
         memset(jobs, 0, sizeof(jobs));
@@ -527,8 +645,9 @@ struct Runner {
         p.carry_in = (d.prenorm && carry_main >= 0) ? scr<float>(P.t_gwhat[carry_main]) : nullptr;
         p.gw_hat = gwhat;
         p.gn0 = gn0;
-        if (P.muon) { p.gxf = scr<float>(P.t_gxf[0]); p.gxb = scr<TN>(P.t_gxb[0]); }
+        if (P.muon) { p.gxf = scr<float>(P.t_gxf[0]); p.gxb = scr<TN>(P.t_gxb[0]); p.gxbt = nullptr; }
         LACT_LAUNCH("k_renorm_bwd", "k_renorm_bwd", 0.0, (k_renorm_bwd<TN>), rowgrid, dim3(256), s, p);
+        if (P.muon && kNsBf16 && P.S > 0) transpose3(scr<TN>(P.t_gxb[0]), gxbt(0), true);
       }
       if (d.prenorm) carry_main = gw_idx;
       if (P.muon) {
@@ -563,7 +682,8 @@ struct Runner {
             p.aux = gf; p.ldaux = c; p.bsaux = xe; p.alpha = 1.f; p.beta = ca;
             p.out = scr<float>(P.t_gxf[cur ^ 1]);
             p.out_c = scr<TN>(P.t_gxb[cur ^ 1]);
-            launch_row_gemm<TN, false, 2, EPI_AXPBY_F32_DUAL>("ns_bwd_gx", p, n, s);
+            const BT bt[2] = {{gxbt(cur), r}, {xbt(u, it), r}};
+            launch_row_gemm<TN, false, 2, EPI_AXPBY_F32_DUAL>("ns_bwd_gx", p, n, s, kNsBf16 ? bt : nullptr, gxbt(cur ^ 1));
           }
           cur ^= 1;
         }
@@ -582,8 +702,10 @@ struct Runner {
         p.m_prev = (P.momentum && u > 0) ? dsave(u - 1) : nullptr;
         p.mbar = P.momentum ? mbar(u) : nullptr;
         p.gc = scr<T>(P.t_gc);
+        p.gct = nullptr;
         p.mdot_part = scr<float>(P.t_mdot);
         LACT_LAUNCH("k_grad_prep", "k_grad_prep", 0.0, (k_grad_prep<T, TN>), dim3(P.nblk, 3 * d.b), dim3(256), s, p);
+        if (kBf16) transpose3(scr<T>(P.t_gc), gct(), false);
         if (P.momentum) {
           gm_valid = true;
           if (u > 0)
@@ -603,8 +725,7 @@ struct Runner {
         hp.lrpart = scr<float>(P.t_lrpart);
         hp.lrpart_stride = (long long)d.b * P.Tcap;
         hp.lrpart_mat_stride = (long long)P.lr_slots * d.b * P.Tcap;
-        dim3 grid(ceil_div(T_, TSB::BM), ceil_div(d.dh, TSB::BN), d.b);
-        LACT_LAUNCH("k_update_bwd_hidden", "update_bwd_hidden", 12.0 * T_ * d.d * d.dh * d.b, (k_update_bwd_hidden<T, TSB>), grid, dim3(TSB::THREADS), s, hp);
+        launch_hidden(3, hp, vprev, gct(1), T_);
       }
       const bool acc_kv = overlaps(seen_kv, st.start, st.end);
       {  // dk = (dgate*lr0) G0 + (dh2*lr2) G2 + gG W0 + gH2 W2
@@ -615,7 +736,8 @@ struct Runner {
         set_term(p.t[3], h(2), d.dh, hbs(), wc(vprev, 2), d.d, P.g.elems, d.dh);
         p.M = T_; p.N = d.d; p.out = dk + (size_t)st.start * d.d; p.ldo = d.d; p.bso = (long long)d.kv_len * d.d;
         p.accumulate = acc_kv;
-        launch_row_gemm<T, false, 4, EPI_STORE>("update_bwd_dk", p, d.b, s);
+        const BT bt[4] = {{gct(0), d.dh}, {gct(2), d.dh}, {wct(vprev, 0), d.dh}, {wct(vprev, 2), d.dh}};
+        launch_row_gemm<T, false, 4, EPI_STORE>("update_bwd_dk", p, d.b, s, kBf16 ? bt : nullptr, nullptr, true);
       }
       {  // dv = (hidden*lr1) G1^T + gDH W1^T
         auto p = row_params<2>();
@@ -623,7 +745,7 @@ struct Runner {
         set_term(p.t[1], h(1), d.dh, hbs(), wc(vprev, 1), d.dh, P.g.elems, d.dh);
         p.M = T_; p.N = d.d; p.out = dv + (size_t)st.start * d.d; p.ldo = d.d; p.bso = (long long)d.kv_len * d.d;
         p.accumulate = acc_kv;
-        launch_row_gemm<T, true, 2, EPI_STORE>("update_bwd_dv", p, d.b, s);
+        launch_row_gemm<T, true, 2, EPI_STORE>("update_bwd_dv", p, d.b, s, nullptr, nullptr, true);
       }
       {
         TokenReduceJob jobs[3];
@@ -640,7 +762,8 @@ struct Runner {
         LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, gwcur, gwhat, pass, partial, sp.n, (long long)P.mat3);
       }
       LACT_LAUNCH("k_lr_reduce", "k_lr_reduce", 0.0, k_lr_reduce, dim3(ceil_div(T_, 256), d.b, 3), dim3(256), s, scr<float>(P.t_lrpart),
-                         (long long)P.lr_slots * d.b * P.Tcap, (long long)d.b * P.Tcap, P.lr_slots, P.Tcap, dlr0, dlr1, dlr2,
+                         (long long)P.lr_slots * d.b * P.Tcap, (long long)d.b * P.Tcap,
+                  kBf16 ? ceil_div(d.dh, TS_BWD::BN) * TS_BWD::WAVES_N : ceil_div(d.dh, TSB::BN) * TSB::WAVES_N, P.Tcap, dlr0, dlr1, dlr2,
                          (long long)d.kv_len, st.start, T_);
       --ver;
     }
@@ -719,6 +842,7 @@ int newton_schulz_t(int32_t n, int32_t rows, int32_t cols, const float* gin, flo
     I.xf_out = last ? nullptr : reinterpret_cast<float*>(ws + P.o_xf[(it + 1) & 1]);
     I.xb_out = last ? nullptr : ws + P.o_xb[(it + 1) & 1];
     I.u_out = last ? out : nullptr;
+    I.xbt_in = nullptr; I.xbt_out = nullptr;
     ns_iteration<TN>(I, s);
   }
   LACT_CHECK_LAUNCH();

@@ -17,6 +17,11 @@ struct MatGeom {
   __host__ __device__ int cols(int j) const { return j == 1 ? dh : d; }
   __host__ __device__ bool tall(int j) const { return rows(j) > cols(j); }
   __host__ __device__ int maxrows() const { return d > dh ? d : dh; }
+  // Newton-Schulz orientation is [r, c] = [min, max]; index of the same element in the [c, r] transpose
+  __device__ long long xtidx(long long x) const {
+    const int r = d < dh ? d : dh, c = d < dh ? dh : d;
+    return (x % c) * r + x / c;
+  }
   // index of original element e = i*cols + j inside the Newton-Schulz orientation
   __device__ long long xidx(int j, long long e) const {
     if (!tall(j)) return e;
@@ -33,6 +38,7 @@ struct InitParams {
   float* n0;              // [3b][maxrows]
   float* wf;              // [3b][elems]
   void* wc;               // [3b][elems] compute type, or null when the compute type is fp32
+  uint16_t* wct;          // [3b][elems] bf16, each matrix transposed ([cols][rows]), or null
 };
 template <typename T>
 __global__ void k_init_state(const InitParams p) {
@@ -48,6 +54,7 @@ __global__ void k_init_state(const InitParams p) {
     ss += v * v;
     dst[c] = v;
     if (p.wc) Elem<T>::store(reinterpret_cast<T*>(p.wc) + (size_t)z * p.g.elems + (size_t)row * cols + c, v);
+    if (p.wct) p.wct[(size_t)z * p.g.elems + (size_t)c * p.g.rows(j) + row] = f32_to_bf16(v);
   }
   ss = wave_sum(ss);
   if (lane == 0) p.n0[(size_t)z * p.g.maxrows() + row] = sqrtf(ss);
@@ -106,6 +113,7 @@ struct NsScaleParams {
   const void* g16; const float* ss_part; int nparts;
   float* norms;          // [3b]
   float* xf; void* xb;   // [3b][elems], Newton-Schulz orientation (fp32 iterate, copy in the Newton-Schulz type)
+  uint16_t* xbt;         // [3b][elems] bf16 copy transposed ([c][r]), or null
   float* u;              // [3b][elems] original orientation, or null (only when zero iterations follow)
   int plain_bf16;        // reference without autocast: norm and quotient are bf16 tensors
 };
@@ -128,6 +136,7 @@ __global__ void k_ns_scale(const NsScaleParams p) {
     if (p.plain_bf16) v = round_bf16(v);
     p.xf[(size_t)z * p.g.elems + x] = v;
     Elem<TN>::store(reinterpret_cast<TN*>(p.xb) + (size_t)z * p.g.elems + x, v);
+    if (p.xbt) p.xbt[(size_t)z * p.g.elems + p.g.xtidx(x)] = f32_to_bf16(v);
     if (p.u) p.u[(size_t)z * p.g.elems + e] = v;
   }
 }
@@ -142,6 +151,8 @@ struct RenormParams {
   int weight_norm;
   float* main_out;                 // un-normalised accumulator (pre-norm) or null
   float* wf_out; void* wc_out;     // new weights: fp32 state and compute-type copy (may be null)
+  uint16_t* wct_out;               // bf16 transposed copy ([cols][rows]) or null
+  uint16_t* gxbt;                  // backward: bf16 transposed copy of the Newton-Schulz-orientation gradient, or null
   // backward only
   const float* gy;                 // gradient w.r.t. the new weights
   const float* carry_in;           // gradient arriving at the accumulator from later steps (pre-norm) or null
@@ -177,6 +188,7 @@ __global__ void k_update_renorm(const RenormParams p) {
     const float y = p.weight_norm ? (v / den) * n0 : v;
     p.wf_out[o + c] = y;
     if (p.wc_out) Elem<T>::store(reinterpret_cast<T*>(p.wc_out) + o + c, y);
+    if (p.wct_out) p.wct_out[(size_t)z * p.g.elems + (size_t)c * p.g.rows(j) + row] = f32_to_bf16(y);
   }
 }
 
@@ -213,6 +225,7 @@ __global__ void k_renorm_bwd(const RenormParams p) {
       const size_t x = (size_t)z * p.g.elems + p.g.xidx(j, (long long)row * cols + c);
       p.gxf[x] = gv;
       Elem<TN>::store(reinterpret_cast<TN*>(p.gxb) + x, gv);
+      if (p.gxbt) p.gxbt[(size_t)z * p.g.elems + p.g.xtidx(x - (size_t)z * p.g.elems)] = f32_to_bf16(gv);
     }
   }
 }
@@ -243,6 +256,7 @@ struct GradPrepParams {
   float* gm_carry; int carry_valid;  // gradient w.r.t. the momentum state after this update (in/out)
   const float* m_prev; const float* mbar;   // null without momentum
   void* gc;                          // [3b][elems] compute-type copy of d loss / d dw  (GEMM operand)
+  uint16_t* gct;                     // bf16 transposed copy ([cols][rows]) or null
   float* mdot_part;                  // [3b][gridDim.x] partial <g, m_prev>
 };
 template <typename T, typename TN>
@@ -277,6 +291,10 @@ __global__ void k_grad_prep(const GradPrepParams p) {
       if (p.m_prev) md += gv * p.m_prev[o];
     }
     Elem<T>::store(reinterpret_cast<T*>(p.gc) + o, gv);
+    if (p.gct) {
+      const int cols = p.g.cols(j);
+      p.gct[(size_t)z * p.g.elems + (e % cols) * p.g.rows(j) + e / cols] = f32_to_bf16(gv);
+    }
   }
   if (p.gm_carry) {
     md = block_sum(md, red);
@@ -356,6 +374,41 @@ __global__ void k_pack3(float* dst, long long elems, int nb, const float* i0, co
   const float* src = (z / nb) == 0 ? i0 : ((z / nb) == 1 ? i1 : i2);
   dst[(size_t)z * elems + e] = src ? src[(size_t)(z % nb) * elems + e] : 0.f;
 }
+// dst[z][c*rows + r] = src[z][r*cols + c] for bf16 matrices; kind j = z / nb picks (rows, cols).
+struct TransposeParams {
+  const uint16_t* src; uint16_t* dst;
+  int rows[3], cols[3];
+  int nb; long long elems;
+};
+__global__ __launch_bounds__(256) void k_transpose_b16(const TransposeParams p) {
+  __shared__ uint16_t tile[64][66];
+  const int z = blockIdx.z, j = z / p.nb;
+  const int rows = p.rows[j], cols = p.cols[j];
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  if (r0 >= rows || c0 >= cols) return;
+  const uint16_t* src = p.src + (size_t)z * p.elems;
+  uint16_t* dst = p.dst + (size_t)z * p.elems;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int idx = threadIdx.x + i * 256, r = idx / 16, c = (idx % 16) * 4;
+    uint2 v = make_uint2(0, 0);
+    if (r0 + r < rows && c0 + c < cols) v = *reinterpret_cast<const uint2*>(src + (size_t)(r0 + r) * cols + c0 + c);
+    tile[r][c] = (uint16_t)(v.x & 0xffff); tile[r][c + 1] = (uint16_t)(v.x >> 16);
+    tile[r][c + 2] = (uint16_t)(v.y & 0xffff); tile[r][c + 3] = (uint16_t)(v.y >> 16);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int idx = threadIdx.x + i * 256, c = idx / 16, r = (idx % 16) * 4;
+    if (c0 + c < cols && r0 + r < rows) {
+      uint2 v;
+      v.x = (uint32_t)tile[r][c] | ((uint32_t)tile[r + 1][c] << 16);
+      v.y = (uint32_t)tile[r + 2][c] | ((uint32_t)tile[r + 3][c] << 16);
+      *reinterpret_cast<uint2*>(dst + (size_t)(c0 + c) * rows + r0 + r) = v;
+    }
+  }
+}
+
 __global__ void k_fill_f32(float* p, float v, long long n) {
   const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (e < n) p[e] = v;
