@@ -37,10 +37,12 @@ __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
+// K-contiguous operand: element (r, k) at base[r*ld + k].  K-strided (ks): element (r, k) at base[k*ld + r].
 struct DmaOperand {
-  const uint16_t* base;  // first row of this block's tile
+  const uint16_t* base;  // first row (r = 0, k = 0) of this block's tile
   int ld;
-  int rows;              // valid rows from base on (may exceed the tile)
+  int rows;              // valid rows from base on (may exceed the tile); multiple of 8 when ks
+  int ks;
 };
 
 // One phase: acc[j] += A * B_j^T over K, j < nb.
@@ -58,25 +60,41 @@ constexpr int DMA_BK = 64;
 // instruction.  Rows past the operand are clamped to its last row: what they bring in only reaches output
 // rows/columns that are never stored.  K must be a multiple of 64 (the host routes other shapes to the
 // generic kernels).
+// K-strided tiles are copied as they lie in memory, [64 k][ROWS] with the 16-byte granules of k-row k rotated
+// by 4*(k % 4) positions, and read back with ds_read_b64_tr_b16: inside each group of 16 lanes, lane i
+// receives element (i & 3) of the 8 bytes addressed by lanes 4j + (i >> 2), j = 0..3 -- i.e. a 4(k) x 16(r)
+// patch comes back transposed, 4 consecutive k of one r per lane.  The rotation makes the four k-rows of a
+// patch land in different bank groups.
 template <int ROWS>
 struct DmaLane {
   static constexpr int N = ROWS / 8;    // copies per K-step
+  static constexpr int G = ROWS / 8;    // granules per k-row of a K-strided tile
   const uint16_t* base;                 // uniform
-  uint32_t voff[N];                     // byte offset of this lane's granule from base at k0 = 0
+  size_t kstride;                       // uniform: elements between K-steps
+  uint32_t voff[N];                     // byte offset of this lane's granule from base at K-step 0
   __device__ __forceinline__ void init(const DmaOperand& op) {
     const int lane = threadIdx.x & 63;
     base = op.base;
+    kstride = op.ks ? (size_t)DMA_BK * op.ld : (size_t)DMA_BK;
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-      const int row = i * 8 + (lane >> 3);
-      const int kv = ((lane & 7) ^ ((row >> 1) & 7)) * 8;
-      const int r = min(row, op.rows - 1);
-      voff[i] = (uint32_t)(((size_t)r * op.ld + kv) * 2);
+      if (op.ks) {
+        const int L = i * 64 + lane, k = L / G, p = L % G;
+        int g = (p + G - (4 * (k & 3)) % G) % G;
+        g = min(g, op.rows / 8 - 1);
+        voff[i] = (uint32_t)(((size_t)k * op.ld + g * 8) * 2);
+      } else {
+        const int row = i * 8 + (lane >> 3);
+        const int kv = ((lane & 7) ^ ((row >> 1) & 7)) * 8;
+        const int r = min(row, op.rows - 1);
+        voff[i] = (uint32_t)(((size_t)r * op.ld + kv) * 2);
+      }
     }
   }
-  __device__ __forceinline__ void issue(int k0, uint32_t lds_tile) const {
+  __device__ __forceinline__ void issue(int kt, uint32_t lds_tile) const {
+    const uint16_t* b = base + kt * kstride;
 #pragma unroll
-    for (int i = 0; i < N; ++i) dma16(base + k0, voff[i], lds_tile + i * 1024);
+    for (int i = 0; i < N; ++i) dma16(b, voff[i], lds_tile + i * 1024);
   }
 };
 
@@ -84,6 +102,43 @@ __device__ __forceinline__ bf16x8 dma_fetch(const char* tile, int row, int kvec)
   const uint4 u = *reinterpret_cast<const uint4*>(tile + row * 128 + ((kvec ^ ((row >> 1) & 7)) << 4));
   return __builtin_bit_cast(bf16x8, u);
 }
+
+// Fragment source of one 32-row MFMA tile: K-contiguous (one ds_read_b128) or K-strided (two transposing reads).
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+template <int ROWS, bool KS>
+struct FragSrc {
+  uint32_t off0, off1;   // per-lane byte offsets at sub-step 0
+  __device__ __forceinline__ void init(int row0) {   // row0: first row of the 32-row tile inside the operand tile
+    const int l = threadIdx.x & 63;
+    if (KS) {
+      constexpr int G = ROWS / 8, RB = ROWS * 2;
+      const int r = row0 + 16 * ((l >> 4) & 1) + 4 * (l & 3);
+      const int p = (r / 8 + (4 * ((l >> 2) & 3)) % G) % G;
+      const int krow = 8 * (l >> 5) + ((l & 15) >> 2);
+      off0 = krow * RB + p * 16 + (l & 1) * 8;
+      off1 = off0 + 4 * RB;
+    } else {
+      const int row = row0 + (l & 31);
+      off0 = row * 128;
+      off1 = (uint32_t)(((row >> 1) & 7) << 4 | (l >> 5) << 16);   // swizzle key and lane half, unpacked in fetch
+    }
+  }
+  __device__ __forceinline__ bf16x8 fetch(const char* tile, int ks) const {
+    if (KS) {
+      constexpr int RB = ROWS * 2;
+      typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+      const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(tile + off0 + ks * 16 * RB));
+      const s16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(tile + off1 + ks * 16 * RB));
+      typedef short s16x8 __attribute__((ext_vector_type(8)));
+      const s16x8 v = {a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
+      return __builtin_bit_cast(bf16x8, v);
+    } else {
+      const int kvec = ks * 2 + (off1 >> 16);
+      const uint4 u = *reinterpret_cast<const uint4*>(tile + off0 + (((kvec << 4) ^ (off1 & 0xffff))));
+      return __builtin_bit_cast(bf16x8, u);
+    }
+  }
+};
 
 template <class TS, int NBMAX, int STAGES>
 struct DmaSmem {
@@ -141,15 +196,18 @@ struct DmaPipe {
     };
     auto issue_stage = [&]() {
       const uint32_t base = lds_addr(smem + (issued % STAGES) * SM::STAGE);
-      const int k0 = ckt * DMA_BK;
-      la.issue(k0, base);
+      la.issue(ckt, base);
 #pragma unroll
       for (int j = 0; j < NBMAX; ++j)
-        if (j < cnb) lb[j].issue(k0, base + SM::A_BYTES + j * SM::B_BYTES);
+        if (j < cnb) lb[j].issue(ckt, base + SM::A_BYTES + j * SM::B_BYTES);
       ++issued;
-      if (++ckt == cnk && cp + 1 < NPH) next_phase();
+      if (++ckt == cnk)
+        while (cp + 1 < NPH) {
+          next_phase();
+          if (cnk > 0) break;
+        }
     };
-    next_phase();
+    do next_phase(); while (cnk == 0 && cp + 1 < NPH);
     for (int i = 0; i < STAGES - 1 && issued < total; ++i) issue_stage();
     for (int kt = 0; kt < total; ++kt) {
       if (kt + STAGES - 2 < total) wait_vmcnt<AHEAD>();
@@ -160,22 +218,26 @@ struct DmaPipe {
   }
 
   // ---- MFMA waves: one phase, nk K-steps into acc[0..NB).  `step` counts K-steps over all phases.
-  template <int NB>
+  template <int NB, bool A_KS = false, bool B_KS = false>
   __device__ __forceinline__ void run_phase(int nk, int& step, f32x16 (&acc)[NB][TS::TM][TS::TN]) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int wm0 = (wave / TS::WAVES_N) * TS::WM + (lane & 31), wn0 = (wave % TS::WAVES_N) * TS::WN + (lane & 31);
+    const int wave = threadIdx.x >> 6;
+    FragSrc<TS::BM, A_KS> sa[TS::TM];
+    FragSrc<TS::BN, B_KS> sb[TS::TN];
+#pragma unroll
+    for (int i = 0; i < TS::TM; ++i) sa[i].init((wave / TS::WAVES_N) * TS::WM + i * 32);
+#pragma unroll
+    for (int n = 0; n < TS::TN; ++n) sb[n].init((wave % TS::WAVES_N) * TS::WN + n * 32);
     for (int kt = 0; kt < nk; ++kt, ++step) {
       __syncthreads();
       const char* st = smem + (step % STAGES) * SM::STAGE;
       bf16x8 fa[2][TS::TM], fb[2][NB][TS::TN];
       auto fetch = [&](int buf, int ks) {
-        const int kvec = ks * 2 + (lane >> 5);
 #pragma unroll
-        for (int i = 0; i < TS::TM; ++i) fa[buf][i] = dma_fetch(st, wm0 + i * 32, kvec);
+        for (int i = 0; i < TS::TM; ++i) fa[buf][i] = sa[i].fetch(st, ks);
 #pragma unroll
         for (int j = 0; j < NB; ++j)
 #pragma unroll
-          for (int n = 0; n < TS::TN; ++n) fb[buf][j][n] = dma_fetch(st + SM::A_BYTES + j * SM::B_BYTES, wn0 + n * 32, kvec);
+          for (int n = 0; n < TS::TN; ++n) fb[buf][j][n] = sb[n].fetch(st + SM::A_BYTES + j * SM::B_BYTES, ks);
       };
       auto mfmas = [&](int buf) {
 #pragma unroll

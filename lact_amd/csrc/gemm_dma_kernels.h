@@ -24,7 +24,8 @@ struct RowGemmDmaParams {
   uint16_t* out_ct;   // DUAL: bf16 transposed copy [N][M] (batch stride = bso), or null
 };
 
-template <class TS, int NT, int EPI>
+// B_KS: the B operands are [K, N] (N contiguous) instead of [N, K].
+template <class TS, int NT, int EPI, bool B_KS>
 __global__ __launch_bounds__(DMA_THREADS) void k_row_gemm_dma(const RowGemmDmaParams<NT> pp) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int STAGES = row_stages<TS>();
@@ -35,9 +36,9 @@ __global__ __launch_bounds__(DMA_THREADS) void k_row_gemm_dma(const RowGemmDmaPa
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     ph[t].a.base = reinterpret_cast<const uint16_t*>(p.t[t].A) + z * p.t[t].bsA + (size_t)m0 * p.t[t].lda;
-    ph[t].a.ld = p.t[t].lda; ph[t].a.rows = p.M - m0;
-    ph[t].b[0].base = reinterpret_cast<const uint16_t*>(p.t[t].B) + z * p.t[t].bsB + (size_t)n0 * p.t[t].ldb;
-    ph[t].b[0].ld = p.t[t].ldb; ph[t].b[0].rows = p.N - n0;
+    ph[t].a.ld = p.t[t].lda; ph[t].a.rows = p.M - m0; ph[t].a.ks = 0;
+    ph[t].b[0].base = reinterpret_cast<const uint16_t*>(p.t[t].B) + z * p.t[t].bsB + (B_KS ? (size_t)n0 : (size_t)n0 * p.t[t].ldb);
+    ph[t].b[0].ld = p.t[t].ldb; ph[t].b[0].rows = p.N - n0; ph[t].b[0].ks = B_KS;
     ph[t].nb = 1;
     ph[t].K = p.t[t].K;
   }
@@ -52,7 +53,7 @@ __global__ __launch_bounds__(DMA_THREADS) void k_row_gemm_dma(const RowGemmDmaPa
   } else {
     int step = 0;
 #pragma unroll
-    for (int t = 0; t < NT; ++t) pipe.template run_phase<1>(p.t[t].K / DMA_BK, step, acc);
+    for (int t = 0; t < NT; ++t) pipe.template run_phase<1, false, B_KS>(p.t[t].K / DMA_BK, step, acc);
   }
   __syncthreads();
   LACT_TS(2);
@@ -180,7 +181,6 @@ __global__ __launch_bounds__(DMA_THREADS) void k_row_gemm_dma(const RowGemmDmaPa
 // ------------------------------------------------------------------------------------------------
 struct HiddenDmaParams {
   HiddenParams h;
-  const void* W1T; const void* G1T;
 };
 
 template <class TS>
@@ -189,6 +189,7 @@ __device__ __forceinline__ DmaOperand token_operand(const void* base, long long 
   o.base = reinterpret_cast<const uint16_t*>(base) + z * bs + (size_t)m0 * ld;
   o.ld = ld;
   o.rows = T - m0;
+  o.ks = 0;
   return o;
 }
 __device__ __forceinline__ DmaOperand weight_operand(const void* base, long long bs, int ld, int z, int n0, int rows) {
@@ -196,6 +197,16 @@ __device__ __forceinline__ DmaOperand weight_operand(const void* base, long long
   o.base = reinterpret_cast<const uint16_t*>(base) + z * bs + (size_t)n0 * ld;
   o.ld = ld;
   o.rows = rows - n0;
+  o.ks = 0;
+  return o;
+}
+// [K, rows] matrix (rows contiguous): the tile starts at column n0
+__device__ __forceinline__ DmaOperand weight_operand_ks(const void* base, long long bs, int ld, int z, int n0, int rows) {
+  DmaOperand o;
+  o.base = reinterpret_cast<const uint16_t*>(base) + z * bs + n0;
+  o.ld = ld;
+  o.rows = rows - n0;
+  o.ks = 1;
   return o;
 }
 
@@ -261,7 +272,7 @@ __device__ __forceinline__ void three_acc_mainloop(const HiddenDmaParams& pp, ch
   ph[0].nb = 2;
   ph[0].K = p.d;
   ph[1].a = token_operand<TS>(p.Y, p.bsy, p.ldy, z, m0, p.T);
-  ph[1].b[0] = weight_operand(pp.W1T, p.bsw, p.d, z, n0, p.dh);
+  ph[1].b[0] = weight_operand_ks(p.W1, p.bsw, p.dh, z, n0, p.dh);   // V * W1: w1 is [d, dh]
   ph[1].b[1] = ph[1].b[0];
   ph[1].nb = 1;
   ph[1].K = p.d;
@@ -275,7 +286,7 @@ __device__ __forceinline__ void three_acc_mainloop(const HiddenDmaParams& pp, ch
   } else {
     int step = 0;
     pipe.template run_phase<2>(nk, step, a02);
-    pipe.template run_phase<1>(nk, step, a1);
+    pipe.template run_phase<1, false, true>(nk, step, a1);
   }
   __syncthreads();
 }
@@ -367,8 +378,8 @@ __global__ __launch_bounds__(DMA_THREADS) void k_update_bwd_hidden_dma(const Hid
   ph[1].b[0] = weight_operand(p.G0, p.bsw, p.d, z, n0, p.dh);
   ph[1].b[1] = weight_operand(p.G2, p.bsw, p.d, z, n0, p.dh);
   ph[2].a = token_operand<TS>(p.Y, p.bsy, p.ldy, z, m0, p.T);
-  ph[2].b[0] = weight_operand(pp.W1T, p.bsw, p.d, z, n0, p.dh);
-  ph[2].b[1] = weight_operand(pp.G1T, p.bsw, p.d, z, n0, p.dh);
+  ph[2].b[0] = weight_operand_ks(p.W1, p.bsw, p.dh, z, n0, p.dh);
+  ph[2].b[1] = weight_operand_ks(p.G1, p.bsw, p.dh, z, n0, p.dh);
   ph[0].K = ph[1].K = ph[2].K = p.d;
   ph[0].nb = ph[1].nb = ph[2].nb = 2;
   const int nk = (p.d + DMA_BK - 1) / DMA_BK;
@@ -382,7 +393,7 @@ __global__ __launch_bounds__(DMA_THREADS) void k_update_bwd_hidden_dma(const Hid
     int step = 0;
     pipe.template run_phase<2>(nk, step, aw);
     pipe.template run_phase<2>(nk, step, ag);
-    pipe.template run_phase<2>(nk, step, ay);
+    pipe.template run_phase<2, false, true>(nk, step, ay);
   }
   __syncthreads();
   using SB = StageTile<TS, 2>;
@@ -435,6 +446,65 @@ __global__ __launch_bounds__(DMA_THREADS) void k_update_bwd_hidden_dma(const Hid
 #pragma unroll
   for (int i = 0; i < 6; ++i)
     copy_out_b16<TS>(smem + i * SB::BYTES, reinterpret_cast<uint16_t*>(outs[i]) + off, p.dh, p.T - m0, p.dh - n0);
+}
+
+// ------------------------------------------------------------------------------------------------
+// k_token_reduce_dma: the three token-reduction GEMMs of one step (see k_token_reduce), both operands
+// K-strided (tokens are the rows of every activation), fp32 partials per token split.
+// ------------------------------------------------------------------------------------------------
+template <class TS>
+__global__ __launch_bounds__(DMA_THREADS) void k_token_reduce_dma(const TokenReduceParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr int STAGES = row_stages<TS>();
+  using Pipe = DmaPipe<TS, 1, 2, STAGES>;
+  const int j = blockIdx.z / p.nb, ib = blockIdx.z % p.nb;
+  const TokenReduceJob& job = p.job[j];
+  const int tiles_n = (job.N + TS::BN - 1) / TS::BN;
+  const int m0 = (blockIdx.x / tiles_n) * TS::BM, n0 = (blockIdx.x % tiles_n) * TS::BN;
+  if (m0 >= job.M) return;
+  const int k_begin = blockIdx.y * p.split_len;
+  const int klen = min(p.split_len, p.tokens - k_begin);
+  DmaPhase<1> ph[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const TokenReduceTerm& tt = job.t[t < job.nterms ? t : 0];
+    ph[t].a.base = reinterpret_cast<const uint16_t*>(tt.A) + ib * tt.bsA + (size_t)k_begin * tt.lda + m0;
+    ph[t].a.ld = tt.lda; ph[t].a.rows = job.M - m0; ph[t].a.ks = 1;
+    ph[t].b[0].base = reinterpret_cast<const uint16_t*>(tt.B) + ib * tt.bsB + (size_t)k_begin * tt.ldb + n0;
+    ph[t].b[0].ld = tt.ldb; ph[t].b[0].rows = job.N - n0; ph[t].b[0].ks = 1;
+    ph[t].nb = 1;
+    ph[t].K = t < job.nterms ? klen : 0;
+  }
+  f32x16 acc[1][TS::TM][TS::TN];
+  zero_acc<TS>(acc[0]);
+  Pipe pipe(smem, ph);
+  const bool loader = Pipe::is_loader();
+  if (loader) {
+    pipe.template load_all<Pipe::loads(1)>();
+  } else {
+    int step = 0;
+    pipe.template run_phase<1, true, true>(ph[0].K / DMA_BK, step, acc);
+    pipe.template run_phase<1, true, true>(ph[1].K / DMA_BK, step, acc);
+  }
+  __syncthreads();
+  using ST = StageTile<TS, 4>;
+  if (!loader) {
+    char* lb = smem + ST::lane_base();
+    LACT_FOR_QUADS(TS) ST::put4(lb, tm, tn, g, acc[0][tm][tn][4 * g], acc[0][tm][tn][4 * g + 1], acc[0][tm][tn][4 * g + 2], acc[0][tm][tn][4 * g + 3]);
+  }
+  __syncthreads();
+  float* out = p.partial + ((size_t)blockIdx.y * gridDim.z + blockIdx.z) * p.mat_elems;
+  const int r0 = ST::row0(), c0 = ST::col0();
+  if (ST::active() && n0 + c0 < job.N) {
+    const char* src = smem + (r0 * ST::LD + c0) * 4;
+    float* dst = out + (size_t)(m0 + r0) * job.N + n0 + c0;
+#pragma unroll
+    for (int ps = 0; ps < ST::PASSES; ++ps) {
+      const int r = r0 + ps * ST::RPP;
+      if (r < TS::BM && m0 + r < job.M) *reinterpret_cast<float4*>(dst) = *reinterpret_cast<const float4*>(src + ps * ST::RPP * ST::LD * 4);
+      dst += (size_t)ST::RPP * job.N;
+    }
+  }
 }
 
 }  // namespace lact

@@ -117,7 +117,7 @@ struct Split {
 Split choose_split(int tokens, int tiles_total) {
   int ns = std::max(1, ceil_div(512, std::max(1, tiles_total)));
   ns = std::min(ns, std::max(1, tokens / 128));
-  int len = ceil_div(ceil_div(tokens, ns), 32) * 32;
+  int len = ceil_div(ceil_div(tokens, ns), 64) * 64;
   return Split{ceil_div(tokens, len), len};
 }
 
@@ -240,43 +240,34 @@ const char* row_gemm_name() {
                                (EPI == EPI_STORE ? ",store>" : (EPI == EPI_AXPBY ? ",axpby>" : ",axpby_dual>"));
   return n.c_str();
 }
-// transposed ([N][K], K contiguous) copy of a K-strided B operand, for the asynchronous-copy kernels
-struct BT {
-  const void* p;
-  int ld;
-};
-template <class TS, int NT, int EPI>
+template <class TS, int NT, int EPI, bool B_KS>
 void launch_row_gemm_dma(const char* site, const RowGemmDmaParams<NT>& q, int batch, hipStream_t s) {
   constexpr int STAGES = row_stages<TS>();
   constexpr int SMEM = cmax(DmaSmem<TS, 1, STAGES>::BYTES, StageTile<TS, 4>::BYTES);
-  static bool once = (allow_big_lds(k_row_gemm_dma<TS, NT, EPI>, SMEM), true);
+  static bool once = (allow_big_lds(k_row_gemm_dma<TS, NT, EPI, B_KS>, SMEM), true);
   (void)once;
   static const std::string name = std::string("k_row_gemm_dma<") + std::to_string(TS::BM) + "x" + std::to_string(TS::BN) + "," +
-                                  std::to_string(NT) + (EPI == EPI_STORE ? ",store>" : (EPI == EPI_AXPBY ? ",axpby>" : ",axpby_dual>"));
+                                  std::to_string(NT) + (EPI == EPI_STORE ? ",store" : (EPI == EPI_AXPBY ? ",axpby" : ",axpby_dual")) +
+                                  (B_KS ? ",Bks>" : ",Bkc>");
   dim3 grid(ceil_div(q.g.M, TS::BM), ceil_div(q.g.N, TS::BN), batch);
   double ksum = 0;
   for (int t = 0; t < NT; ++t) ksum += q.g.t[t].K;
-  LACT_LAUNCH_SMEM(name.c_str(), site, 2.0 * q.g.M * q.g.N * ksum * batch, (k_row_gemm_dma<TS, NT, EPI>), grid, dim3(DMA_THREADS),
-                   SMEM, s, q);
+  LACT_LAUNCH_SMEM(name.c_str(), site, 2.0 * q.g.M * q.g.N * ksum * batch, (k_row_gemm_dma<TS, NT, EPI, B_KS>), grid,
+                   dim3(DMA_THREADS), SMEM, s, q);
 }
+// bf16 with every K a multiple of 64: asynchronous-copy kernels; anything else: the generic tile loop
 template <typename T, bool B_KC, int NT, int EPI>
-void launch_row_gemm(const char* site, const RowGemmParams<NT>& p, int batch, hipStream_t s, const BT* bt = nullptr,
-                     uint16_t* out_ct = nullptr, bool token_rows = false) {
+void launch_row_gemm(const char* site, const RowGemmParams<NT>& p, int batch, hipStream_t s, bool token_rows = false) {
   if constexpr (std::is_same<T, uint16_t>::value) {
-    bool k64 = true;
-    for (int t = 0; t < NT; ++t) k64 = k64 && p.t[t].K % 64 == 0;
-    if ((B_KC || bt) && k64) {
+    bool ok = p.N % 8 == 0;
+    for (int t = 0; t < NT; ++t) ok = ok && p.t[t].K % 64 == 0;
+    if (ok) {
       RowGemmDmaParams<NT> q;
       q.g = p;
-      q.out_ct = out_ct;
-      if (!B_KC)
-        for (int t = 0; t < NT; ++t) {
-          q.g.t[t].B = bt[t].p;
-          q.g.t[t].ldb = bt[t].ld;
-        }
-      if (token_rows) launch_row_gemm_dma<TS_ROW, NT, EPI>(site, q, batch, s);
-      else if (p.M % TS_NS::BM == 0 && p.N % TS_NS::BN == 0) launch_row_gemm_dma<TS_NS, NT, EPI>(site, q, batch, s);
-      else launch_row_gemm_dma<TS_SQ, NT, EPI>(site, q, batch, s);
+      q.out_ct = nullptr;
+      if (token_rows) launch_row_gemm_dma<TS_ROW, NT, EPI, !B_KC>(site, q, batch, s);
+      else if (p.M % TS_NS::BM == 0 && p.N % TS_NS::BN == 0) launch_row_gemm_dma<TS_NS, NT, EPI, !B_KC>(site, q, batch, s);
+      else launch_row_gemm_dma<TS_SQ, NT, EPI, !B_KC>(site, q, batch, s);
       return;
     }
   }
@@ -310,7 +301,6 @@ struct NsIter {
   const float* xf_in; const void* xb_in;           // X: fp32 iterate and its copy in the GEMM type
   void* ab; void* bb;                              // A and B of this iteration (GEMM type)
   float* xf_out; void* xb_out; float* u_out;       // X': fp32, GEMM type, and fp32 in the original orientation (each nullable)
-  const uint16_t* xbt_in; uint16_t* xbt_out;       // bf16 [c][r] copies of X and X' (asynchronous-copy kernels), nullable
 };
 // TN: GEMM operand type of the iteration (bf16 as in the reference, or fp32 for the exact mode)
 template <typename TN>
@@ -337,8 +327,7 @@ void ns_iteration(const NsIter& I, hipStream_t s) {
     p.round_out_bf16 = I.plain;
     p.out = I.xf_out; p.out_c = I.xb_out; p.out_t = I.u_out;
     p.transpose_mask = I.mask; p.nb = I.nb_for_mask;
-    const BT bt[1] = {{I.xbt_in, I.r}};
-    launch_row_gemm<TN, false, 1, EPI_AXPBY_F32_DUAL>("ns_next", p, I.n, s, I.xbt_in ? bt : nullptr, I.xbt_out);
+    launch_row_gemm<TN, false, 1, EPI_AXPBY_F32_DUAL>("ns_next", p, I.n, s);
   }
 }
 
@@ -395,14 +384,13 @@ struct Runner {
   }
 
   // the four hidden-layer kernels: asynchronous-copy version for bf16, generic tile loop otherwise
-  void launch_hidden(int which, const HiddenParams& hp, int ver, const uint16_t* g1t, int T_) const {
+  void launch_hidden(int which, const HiddenParams& hp, int ver, int T_) const {
     const double f = (double)T_ * d.d * d.dh * d.b;
     if (kBf16 && d.d % 64 == 0) {
       if constexpr (kBf16) {
       HiddenDmaParams q;
       q.h = hp;
-      q.W1T = wct(ver, 1);
-      q.G1T = g1t;
+      (void)ver;
       constexpr int SM3 = cmax(DmaSmem<TS_SQ, 2, 3>::BYTES, 3 * StageTile<TS_SQ, 2>::BYTES);
       constexpr int SM6 = cmax(DmaSmem<TS_BWD, 2, 3>::BYTES, 6 * StageTile<TS_BWD, 2>::BYTES);
       dim3 g3(ceil_div(T_, TS_SQ::BM), ceil_div(d.dh, TS_SQ::BN), d.b), g6(ceil_div(T_, TS_BWD::BM), ceil_div(d.dh, TS_BWD::BN), d.b);
@@ -445,6 +433,27 @@ struct Runner {
     for (int i = 0; i < 3; ++i) p.job[i] = jobs[i];
     p.nb = d.b; p.tokens = tokens; p.split_len = sp.len;
     p.partial = scr<float>(P.t_partial); p.mat_elems = P.g.elems;
+    if constexpr (kBf16) {
+      if (sp.len % 64 == 0 && tokens % 64 == 0 && d.d % 8 == 0 && d.dh % 8 == 0) {
+        const bool big = d.d % TS_NS::BM == 0 && d.dh % TS_NS::BM == 0;
+        const int tiles = big ? (d.d / TS_NS::BM) * (d.dh / TS_NS::BN)
+                              : std::max(ceil_div(d.dh, TS_SQ::BM) * ceil_div(d.d, TS_SQ::BN), ceil_div(d.d, TS_SQ::BM) * ceil_div(d.dh, TS_SQ::BN));
+        dim3 g(tiles, sp.n, 3 * d.b);
+        const double fl = 6.0 * tokens * d.d * d.dh * d.b * jobs[0].nterms;
+        if (big) {
+          constexpr int SM = cmax(DmaSmem<TS_NS, 1, row_stages<TS_NS>()>::BYTES, StageTile<TS_NS, 4>::BYTES);
+          static bool once = (allow_big_lds(k_token_reduce_dma<TS_NS>, SM), true);
+          (void)once;
+          LACT_LAUNCH_SMEM("k_token_reduce_dma<192x192>", site, fl, (k_token_reduce_dma<TS_NS>), g, dim3(DMA_THREADS), SM, s, p);
+        } else {
+          constexpr int SM = cmax(DmaSmem<TS_SQ, 1, row_stages<TS_SQ>()>::BYTES, StageTile<TS_SQ, 4>::BYTES);
+          static bool once = (allow_big_lds(k_token_reduce_dma<TS_SQ>, SM), true);
+          (void)once;
+          LACT_LAUNCH_SMEM("k_token_reduce_dma<128x128>", site, fl, (k_token_reduce_dma<TS_SQ>), g, dim3(DMA_THREADS), SM, s, p);
+        }
+        return;
+      }
+    }
     dim3 grid(P.tiles, sp.n, 3 * d.b);
     LACT_LAUNCH("k_token_reduce", site, 6.0 * tokens * d.d * d.dh * d.b * jobs[0].nterms, (k_token_reduce<T, TSA>), grid, dim3(TSA::THREADS), s, p);
   }
@@ -474,7 +483,6 @@ struct Runner {
       p.wc = P.bf16 ? (void*)wc(0) : nullptr;
       p.wct = nullptr;
       LACT_LAUNCH("k_init_state", "k_init_state", 0.0, (k_init_state<T>), rowgrid, dim3(256), s, p);
-      if (kBf16) transpose3(wc(0), wct(0), false);
     }
     int ver = 0, u = 0;
     for (const auto& st : P.steps) {
@@ -482,11 +490,11 @@ struct Runner {
       if (st.kind == LACT_APPLY) {
         HiddenParams hp = hidden_params(T_, q + (size_t)st.start * d.q_ld, d.q_ld, d.q_bs, nullptr, 0, 0, ver);
         hp.O0 = h(0);
-        launch_hidden(0, hp, ver, nullptr, T_);
+        launch_hidden(0, hp, ver, T_);
         auto p = row_params<1>();
         set_term(p.t[0], h(0), d.dh, hbs(), wc(ver, 1), d.dh, P.g.elems, d.dh);
         p.M = T_; p.N = d.d; p.out = out + (size_t)st.out_start * d.o_ld; p.ldo = d.o_ld; p.bso = d.o_bs;
-        launch_row_gemm<T, true, 1, EPI_STORE>("apply_out", p, d.b, s, nullptr, nullptr, true);
+        launch_row_gemm<T, true, 1, EPI_STORE>("apply_out", p, d.b, s, true);
         continue;
       }
       // ---- update
@@ -496,7 +504,7 @@ struct Runner {
         HiddenParams hp = hidden_params(T_, kc, d.k_ld, d.k_bs, vc, d.v_ld, d.v_bs, ver);
         hp.lr0 = lr0 + st.start; hp.lr1 = lr1 + st.start; hp.lr2 = lr2 + st.start; hp.bslr = d.kv_len;
         hp.O0 = h(0); hp.O1 = h(1); hp.O2 = h(2);
-        launch_hidden(1, hp, ver, nullptr, T_);
+        launch_hidden(1, hp, ver, T_);
       }
       const Split sp = choose_split(T_, P.tiles * 3 * d.b);
       {
@@ -533,7 +541,6 @@ struct Runner {
         p.u = P.S == 0 ? usave(u) : nullptr;
         p.plain_bf16 = d.ns_mode == LACT_NS_PLAIN_BF16;
         LACT_LAUNCH("k_ns_scale", "k_ns_scale", 0.0, (k_ns_scale<TN>), dim3(P.nblk, 3 * d.b), dim3(256), s, p);
-        if (kNsBf16 && P.S > 0) transpose3(xb(u, 0), xbt(u, 0), true);
         for (int it = 0; it < P.S; ++it) {
           const bool last = it + 1 == P.S;
           NsIter I;
@@ -544,7 +551,6 @@ struct Runner {
           I.xf_out = last ? nullptr : scr<float>(P.t_xf[(it + 1) & 1]);
           I.xb_out = last ? (void*)scr<TN>(P.t_xbtmp) : (void*)xb(u, it + 1);
           I.u_out = last ? usave(u) : nullptr;
-          I.xbt_in = xbt(u, it); I.xbt_out = last ? nullptr : xbt(u, it + 1);
           ns_iteration<TN>(I, s);
         }
       }
@@ -555,7 +561,6 @@ struct Runner {
         p.wc_out = P.bf16 ? (void*)wc(ver + 1) : nullptr;
         p.wct_out = nullptr;
         LACT_LAUNCH("k_update_renorm", "k_update_renorm", 0.0, (k_update_renorm<T>), rowgrid, dim3(256), s, p);
-        if (kBf16) transpose3(wc(ver + 1), wct(ver + 1), false);
       }
       ++ver;
       ++u;
@@ -610,15 +615,14 @@ struct Runner {
         const T* gc = dout + (size_t)st.out_start * d.do_ld;
         HiddenParams hp = hidden_params(T_, qc, d.q_ld, d.q_bs, gc, d.do_ld, d.do_bs, ver);
         hp.O0 = h(0); hp.O1 = h(1); hp.O2 = h(2);
-        launch_hidden(2, hp, ver, nullptr, T_);
+        launch_hidden(2, hp, ver, T_);
         {  // dq = gY0 W0 + gY2 W2
           auto p = row_params<2>();
           set_term(p.t[0], h(1), d.dh, hbs(), wc(ver, 0), d.d, P.g.elems, d.dh);
           set_term(p.t[1], h(2), d.dh, hbs(), wc(ver, 2), d.d, P.g.elems, d.dh);
           p.M = T_; p.N = d.d; p.out = dq + (size_t)st.start * d.d; p.ldo = d.d; p.bso = (long long)d.q_len * d.d;
           p.accumulate = overlaps(seen_q, st.start, st.end);
-          const BT bt[2] = {{wct(ver, 0), d.dh}, {wct(ver, 2), d.dh}};
-          launch_row_gemm<T, false, 2, EPI_STORE>("apply_bwd_dq", p, d.b, s, kBf16 ? bt : nullptr, nullptr, true);
+          launch_row_gemm<T, false, 2, EPI_STORE>("apply_bwd_dq", p, d.b, s, true);
         }
         TokenReduceJob jobs[3];
         memset(jobs, 0, sizeof(jobs));
@@ -647,7 +651,6 @@ struct Runner {
         p.gn0 = gn0;
         if (P.muon) { p.gxf = scr<float>(P.t_gxf[0]); p.gxb = scr<TN>(P.t_gxb[0]); p.gxbt = nullptr; }
         LACT_LAUNCH("k_renorm_bwd", "k_renorm_bwd", 0.0, (k_renorm_bwd<TN>), rowgrid, dim3(256), s, p);
-        if (P.muon && kNsBf16 && P.S > 0) transpose3(scr<TN>(P.t_gxb[0]), gxbt(0), true);
       }
       if (d.prenorm) carry_main = gw_idx;
       if (P.muon) {
@@ -682,8 +685,7 @@ struct Runner {
             p.aux = gf; p.ldaux = c; p.bsaux = xe; p.alpha = 1.f; p.beta = ca;
             p.out = scr<float>(P.t_gxf[cur ^ 1]);
             p.out_c = scr<TN>(P.t_gxb[cur ^ 1]);
-            const BT bt[2] = {{gxbt(cur), r}, {xbt(u, it), r}};
-            launch_row_gemm<TN, false, 2, EPI_AXPBY_F32_DUAL>("ns_bwd_gx", p, n, s, kNsBf16 ? bt : nullptr, gxbt(cur ^ 1));
+            launch_row_gemm<TN, false, 2, EPI_AXPBY_F32_DUAL>("ns_bwd_gx", p, n, s);
           }
           cur ^= 1;
         }
@@ -705,7 +707,6 @@ struct Runner {
         p.gct = nullptr;
         p.mdot_part = scr<float>(P.t_mdot);
         LACT_LAUNCH("k_grad_prep", "k_grad_prep", 0.0, (k_grad_prep<T, TN>), dim3(P.nblk, 3 * d.b), dim3(256), s, p);
-        if (kBf16) transpose3(scr<T>(P.t_gc), gct(), false);
         if (P.momentum) {
           gm_valid = true;
           if (u > 0)
@@ -725,7 +726,7 @@ struct Runner {
         hp.lrpart = scr<float>(P.t_lrpart);
         hp.lrpart_stride = (long long)d.b * P.Tcap;
         hp.lrpart_mat_stride = (long long)P.lr_slots * d.b * P.Tcap;
-        launch_hidden(3, hp, vprev, gct(1), T_);
+        launch_hidden(3, hp, vprev, T_);
       }
       const bool acc_kv = overlaps(seen_kv, st.start, st.end);
       {  // dk = (dgate*lr0) G0 + (dh2*lr2) G2 + gG W0 + gH2 W2
@@ -736,8 +737,7 @@ struct Runner {
         set_term(p.t[3], h(2), d.dh, hbs(), wc(vprev, 2), d.d, P.g.elems, d.dh);
         p.M = T_; p.N = d.d; p.out = dk + (size_t)st.start * d.d; p.ldo = d.d; p.bso = (long long)d.kv_len * d.d;
         p.accumulate = acc_kv;
-        const BT bt[4] = {{gct(0), d.dh}, {gct(2), d.dh}, {wct(vprev, 0), d.dh}, {wct(vprev, 2), d.dh}};
-        launch_row_gemm<T, false, 4, EPI_STORE>("update_bwd_dk", p, d.b, s, kBf16 ? bt : nullptr, nullptr, true);
+        launch_row_gemm<T, false, 4, EPI_STORE>("update_bwd_dk", p, d.b, s, true);
       }
       {  // dv = (hidden*lr1) G1^T + gDH W1^T
         auto p = row_params<2>();
@@ -745,7 +745,7 @@ struct Runner {
         set_term(p.t[1], h(1), d.dh, hbs(), wc(vprev, 1), d.dh, P.g.elems, d.dh);
         p.M = T_; p.N = d.d; p.out = dv + (size_t)st.start * d.d; p.ldo = d.d; p.bso = (long long)d.kv_len * d.d;
         p.accumulate = acc_kv;
-        launch_row_gemm<T, true, 2, EPI_STORE>("update_bwd_dv", p, d.b, s, nullptr, nullptr, true);
+        launch_row_gemm<T, true, 2, EPI_STORE>("update_bwd_dv", p, d.b, s, true);
       }
       {
         TokenReduceJob jobs[3];
@@ -842,7 +842,6 @@ int newton_schulz_t(int32_t n, int32_t rows, int32_t cols, const float* gin, flo
     I.xf_out = last ? nullptr : reinterpret_cast<float*>(ws + P.o_xf[(it + 1) & 1]);
     I.xb_out = last ? nullptr : ws + P.o_xb[(it + 1) & 1];
     I.u_out = last ? out : nullptr;
-    I.xbt_in = nullptr; I.xbt_out = nullptr;
     ns_iteration<TN>(I, s);
   }
   LACT_CHECK_LAUNCH();
