@@ -88,8 +88,8 @@ int lact_forward(const lact_desc_t* desc, const float* w0, const float* w1, cons
  * lact_triton_kernels/lact_swiglu_ffn.py:46-76, lact_fw_grad.py:61-156, l2norm_triton_kernels.py:106-172).
  * dout: gradient of `out` (act_dtype, strides do_ld/do_bs); dw_final[3]: gradient of the returned
  * final weights (nullable).  Outputs: dw0,dw1,dw2 fp32; dq,dk,dv act_dtype contiguous [b,len,d];
- * dlr0..2, dmomentum fp32 [b,kv_len].  dq, dk, dv, dlr*, dmomentum must be zero-filled by the caller
- * (rows no step touches stay zero; rows used by several steps accumulate). */
+ * dlr0..2, dmomentum fp32 [b,kv_len].  Every element of every output is written: rows no step touches
+ * are set to zero, rows used by several steps hold the sum; the caller need not clear anything. */
 int lact_backward(const lact_desc_t* desc, const void* q, const void* k, const void* v, const float* lr0,
                   const float* lr1, const float* lr2, const float* momentum, const void* dout,
                   const float* const dw_final[3], const void* saved, void* scratch, float* dw0, float* dw1,

@@ -493,16 +493,34 @@ __global__ __launch_bounds__(DMA_THREADS) void k_token_reduce_dma(const TokenRed
     LACT_FOR_QUADS(TS) ST::put4(lb, tm, tn, g, acc[0][tm][tn][4 * g], acc[0][tm][tn][4 * g + 1], acc[0][tm][tn][4 * g + 2], acc[0][tm][tn][4 * g + 3]);
   }
   __syncthreads();
-  float* out = p.partial + ((size_t)blockIdx.y * gridDim.z + blockIdx.z) * p.mat_elems;
+  const size_t slot = (size_t)blockIdx.z * p.mat_elems;
+  float* out = p.add_out ? p.add_out + slot : p.partial + (size_t)blockIdx.y * gridDim.z * p.mat_elems + slot;
   const int r0 = ST::row0(), c0 = ST::col0();
   if (ST::active() && n0 + c0 < job.N) {
     const char* src = smem + (r0 * ST::LD + c0) * 4;
-    float* dst = out + (size_t)(m0 + r0) * job.N + n0 + c0;
+    const size_t e0 = (size_t)(m0 + r0) * job.N + n0 + c0, rstep = (size_t)ST::RPP * job.N;
+    float* dst = out + e0;
+    const bool blend = p.add_out && p.add_in;
+    float4 x4[ST::PASSES];
+    if (blend) {
+      const float* ain = p.add_in + slot + e0;
+#pragma unroll
+      for (int ps = 0; ps < ST::PASSES; ++ps) {
+        const int r = r0 + ps * ST::RPP;
+        x4[ps] = (r < TS::BM && m0 + r < job.M) ? *reinterpret_cast<const float4*>(ain + ps * rstep) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    }
 #pragma unroll
     for (int ps = 0; ps < ST::PASSES; ++ps) {
       const int r = r0 + ps * ST::RPP;
-      if (r < TS::BM && m0 + r < job.M) *reinterpret_cast<float4*>(dst) = *reinterpret_cast<const float4*>(src + ps * ST::RPP * ST::LD * 4);
-      dst += (size_t)ST::RPP * job.N;
+      if (r < TS::BM && m0 + r < job.M) {
+        float4 v = *reinterpret_cast<const float4*>(src + ps * ST::RPP * ST::LD * 4);
+        if (blend) {
+          v.x += p.coeff * x4[ps].x; v.y += p.coeff * x4[ps].y; v.z += p.coeff * x4[ps].z; v.w += p.coeff * x4[ps].w;
+        }
+        *reinterpret_cast<float4*>(dst) = v;
+      }
+      dst += rstep;
     }
   }
 }

@@ -342,6 +342,8 @@ struct TokenReduceParams {
   TokenReduceJob job[3];
   int nb, tokens, split_len;   // split_len: tokens per split (multiple of 32)
   float* partial; long long mat_elems;
+  // single split only (asynchronous-copy kernel): out = coeff*add_in + result written here instead of a partial
+  float* add_out; const float* add_in; float coeff;
 };
 
 template <typename T, class TS>

@@ -115,7 +115,8 @@ struct Split {
   int n, len;
 };
 Split choose_split(int tokens, int tiles_total) {
-  int ns = std::max(1, ceil_div(512, std::max(1, tiles_total)));
+  // one split once the tiles alone occupy most of the 256 compute units: the partial sums then never exist
+  int ns = tiles_total >= 160 ? 1 : std::max(1, ceil_div(512, std::max(1, tiles_total)));
   ns = std::min(ns, std::max(1, tokens / 128));
   int len = ceil_div(ceil_div(tokens, ns), 64) * 64;
   return Split{ceil_div(tokens, len), len};
@@ -427,7 +428,10 @@ struct Runner {
     return p;
   }
 
-  void token_reduce(const char* site, const TokenReduceJob (&jobs)[3], int tokens, Split sp) const {
+  // Returns true when the result went straight to `add_out` (= coeff*add_in + sum; single split on the
+  // asynchronous-copy kernel); otherwise the partials are in the scratch slots and the caller reduces them.
+  bool token_reduce(const char* site, const TokenReduceJob (&jobs)[3], int tokens, Split sp, float* add_out = nullptr,
+                    const float* add_in = nullptr, float coeff = 0.f) const {
     TokenReduceParams p;
     memset(&p, 0, sizeof(p));
     for (int i = 0; i < 3; ++i) p.job[i] = jobs[i];
@@ -440,6 +444,8 @@ struct Runner {
                               : std::max(ceil_div(d.dh, TS_SQ::BM) * ceil_div(d.d, TS_SQ::BN), ceil_div(d.d, TS_SQ::BM) * ceil_div(d.dh, TS_SQ::BN));
         dim3 g(tiles, sp.n, 3 * d.b);
         const double fl = 6.0 * tokens * d.d * d.dh * d.b * jobs[0].nterms;
+        const bool direct = add_out && sp.n == 1;
+        if (direct) { p.add_out = add_out; p.add_in = coeff != 0.f ? add_in : nullptr; p.coeff = coeff; }
         if (big) {
           constexpr int SM = cmax(DmaSmem<TS_NS, 1, row_stages<TS_NS>()>::BYTES, StageTile<TS_NS, 4>::BYTES);
           static bool once = (allow_big_lds(k_token_reduce_dma<TS_NS>, SM), true);
@@ -451,11 +457,12 @@ struct Runner {
           (void)once;
           LACT_LAUNCH_SMEM("k_token_reduce_dma<128x128>", site, fl, (k_token_reduce_dma<TS_SQ>), g, dim3(DMA_THREADS), SM, s, p);
         }
-        return;
+        return direct;
       }
     }
     dim3 grid(P.tiles, sp.n, 3 * d.b);
     LACT_LAUNCH("k_token_reduce", site, 6.0 * tokens * d.d * d.dh * d.b * jobs[0].nterms, (k_token_reduce<T, TSA>), grid, dim3(TSA::THREADS), s, p);
+    return false;
   }
 
   RenormParams renorm_params(int u, int ver_prev) const {
@@ -580,12 +587,57 @@ struct Runner {
   }
 
   // ------------------------------------------------------------------------------------------
-  static bool overlaps(std::vector<std::pair<int, int>>& seen, int a, int b) {
-    bool hit = false;
-    for (auto& iv : seen) hit = hit || (a < iv.second && iv.first < b);
-    seen.emplace_back(a, b);
-    return hit;
+  // Gradient rows of a token range are stored on first touch and accumulated on a repeat.  `force` (set when two
+  // ranges of the program overlap without being equal) pre-zeroes the whole buffer and accumulates everywhere.
+  struct Touched {
+    std::vector<std::pair<int, int>> seen;
+    bool force = false;
+    bool accumulate(int a, int b) {
+      bool hit = force;
+      for (auto& iv : seen) hit = hit || (a < iv.second && iv.first < b);
+      seen.emplace_back(a, b);
+      return hit;
+    }
+  };
+  // Rows of [0, len) that no step of `kind` touches, and whether any two of its ranges overlap partially.
+  static std::vector<std::pair<int, int>> untouched(const std::vector<lact_step_t>& steps, int kind, int len, bool* partial) {
+    std::vector<std::pair<int, int>> iv;
+    for (auto& st : steps)
+      if (st.kind == kind) iv.emplace_back(st.start, st.end);
+    *partial = false;
+    for (size_t i = 0; i < iv.size(); ++i)
+      for (size_t j = i + 1; j < iv.size(); ++j)
+        if (iv[i] != iv[j] && iv[i].first < iv[j].second && iv[j].first < iv[i].second) *partial = true;
+    std::sort(iv.begin(), iv.end());
+    std::vector<std::pair<int, int>> gaps;
+    int pos = 0;
+    for (auto& r : iv) {
+      if (r.first > pos) gaps.emplace_back(pos, r.first);
+      pos = std::max(pos, r.second);
+    }
+    if (pos < len) gaps.emplace_back(pos, len);
+    if (*partial) gaps.assign(1, std::make_pair(0, len));
+    return gaps;
   }
+  struct ZeroList {
+    ZeroSegments z;
+    int n = 0;
+    long long maxlen = 0;
+    int nb;
+    hipStream_t s;
+    ZeroList(int nb_, hipStream_t s_) : nb(nb_), s(s_) {}
+    void flush() {
+      if (n > 0 && maxlen > 0)
+        LACT_LAUNCH("k_zero_segments", "k_zero_segments", 0.0, k_zero_segments, dim3((unsigned)((maxlen + 4095) / 4096), nb, n), dim3(256), s, z);
+      n = 0; maxlen = 0;
+    }
+    void add(void* ptr, long long bs, long long off, long long len) {
+      if (!ptr || len <= 0) return;
+      z.ptr[n] = static_cast<char*>(ptr); z.bs[n] = bs; z.off[n] = off; z.len[n] = len;
+      maxlen = std::max(maxlen, len);
+      if (++n == 16) flush();
+    }
+  };
 
   int backward(const T* q, const T* k, const T* v, const float* lr0, const float* lr1, const float* lr2, const float* mom,
                const T* dout, const float* const dwf[3], float* dw0, float* dw1, float* dw2, T* dq, T* dk, T* dv, float* dlr0,
@@ -602,7 +654,21 @@ struct Runner {
     LACT_LAUNCH("k_fill_f32", "k_fill_f32", 0.0, k_fill_f32, dim3((unsigned)((gn0_n + 255) / 256)), dim3(256), s, gn0, 0.f, gn0_n);
     LACT_LAUNCH("k_pack3", "k_pack3", 0.0, k_pack3, eg, dim3(256), s, gwcur, P.g.elems, d.b, dwf ? dwf[0] : nullptr, dwf ? dwf[1] : nullptr,
                        dwf ? dwf[2] : nullptr);
-    std::vector<std::pair<int, int>> seen_q, seen_kv;
+    // every gradient output is written in full by this call: rows that no step touches are zeroed here
+    Touched seen_q, seen_kv;
+    {
+      ZeroList zl(d.b, s);
+      const long long rowb = (long long)d.d * sizeof(T);
+      for (auto& gp : untouched(P.steps, LACT_APPLY, d.q_len, &seen_q.force))
+        zl.add(dq, (long long)d.q_len * rowb, gp.first * rowb, (gp.second - gp.first) * rowb);
+      for (auto& gp : untouched(P.steps, LACT_UPDATE, d.kv_len, &seen_kv.force)) {
+        zl.add(dk, (long long)d.kv_len * rowb, gp.first * rowb, (gp.second - gp.first) * rowb);
+        zl.add(dv, (long long)d.kv_len * rowb, gp.first * rowb, (gp.second - gp.first) * rowb);
+      }
+      float* small[4] = {dlr0, dlr1, dlr2, dmom};
+      for (float* ptr : small) zl.add(ptr, (long long)d.kv_len * 4, 0, (long long)d.kv_len * 4);
+      zl.flush();
+    }
     int ver = P.nupd, u = P.nupd;
     int carry_main = -1;       // index of the gwhat buffer holding the accumulator's gradient (pre-norm)
     bool gm_valid = false;     // gmcarry holds d loss / d (momentum state after update u-1)
@@ -621,7 +687,7 @@ struct Runner {
           set_term(p.t[0], h(1), d.dh, hbs(), wc(ver, 0), d.d, P.g.elems, d.dh);
           set_term(p.t[1], h(2), d.dh, hbs(), wc(ver, 2), d.d, P.g.elems, d.dh);
           p.M = T_; p.N = d.d; p.out = dq + (size_t)st.start * d.d; p.ldo = d.d; p.bso = (long long)d.q_len * d.d;
-          p.accumulate = overlaps(seen_q, st.start, st.end);
+          p.accumulate = seen_q.accumulate(st.start, st.end);
           launch_row_gemm<T, false, 2, EPI_STORE>("apply_bwd_dq", p, d.b, s, true);
         }
         TokenReduceJob jobs[3];
@@ -633,8 +699,8 @@ struct Runner {
         set_tr_term(jobs[1].t[0], gc, d.do_ld, d.do_bs, h(0), d.dh, hbs());
         jobs[2].M = d.dh; jobs[2].N = d.d;
         set_tr_term(jobs[2].t[0], h(2), d.dh, hbs(), qc, d.q_ld, d.q_bs);
-        token_reduce("apply_bwd_dw", jobs, T_, sp);
-        LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, gwcur, gwcur, 1.f, partial, sp.n, (long long)P.mat3);
+        if (!token_reduce("apply_bwd_dw", jobs, T_, sp, gwcur, gwcur, 1.f))
+          LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, gwcur, gwcur, 1.f, partial, sp.n, (long long)P.mat3);
         continue;
       }
       // ---- update u-1: weights ver-1 -> ver
@@ -728,7 +794,7 @@ struct Runner {
         hp.lrpart_mat_stride = (long long)P.lr_slots * d.b * P.Tcap;
         launch_hidden(3, hp, vprev, T_);
       }
-      const bool acc_kv = overlaps(seen_kv, st.start, st.end);
+      const bool acc_kv = seen_kv.accumulate(st.start, st.end);
       {  // dk = (dgate*lr0) G0 + (dh2*lr2) G2 + gG W0 + gH2 W2
         auto p = row_params<4>();
         set_term(p.t[0], h(3), d.dh, hbs(), g0, d.d, P.g.elems, d.dh);
@@ -757,9 +823,9 @@ struct Runner {
         set_tr_term(jobs[1].t[0], vc, d.v_ld, d.v_bs, h(1), d.dh, hbs());
         jobs[2].M = d.dh; jobs[2].N = d.d;
         set_tr_term(jobs[2].t[0], h(2), d.dh, hbs(), kc, d.k_ld, d.k_bs);
-        token_reduce("update_bwd_dw", jobs, T_, sp);
         const float pass = d.prenorm ? 0.f : ((P.muon && d.muon_replaces_weight) ? 0.f : 1.f);
-        LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, gwcur, gwhat, pass, partial, sp.n, (long long)P.mat3);
+        if (!token_reduce("update_bwd_dw", jobs, T_, sp, gwcur, gwhat, pass))
+          LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, gwcur, gwhat, pass, partial, sp.n, (long long)P.mat3);
       }
       LACT_LAUNCH("k_lr_reduce", "k_lr_reduce", 0.0, k_lr_reduce, dim3(ceil_div(T_, 256), d.b, 3), dim3(256), s, scr<float>(P.t_lrpart),
                          (long long)P.lr_slots * d.b * P.Tcap, (long long)d.b * P.Tcap,

@@ -409,6 +409,24 @@ __global__ __launch_bounds__(256) void k_transpose_b16(const TransposeParams p) 
   }
 }
 
+// Zero up to 16 strided byte ranges in one launch: segment i covers, for every batch ib < nb, the bytes
+// [ptr + ib*bs + off, +len); everything a multiple of 4 bytes.  Grid (chunks of 4 KiB, nb, segments).
+struct ZeroSegments {
+  char* ptr[16];
+  long long bs[16], off[16], len[16];
+};
+__global__ void k_zero_segments(const ZeroSegments z) {
+  const int i = blockIdx.z;
+  const long long e = ((long long)blockIdx.x * blockDim.x + threadIdx.x) * 16;
+  if (e >= z.len[i]) return;
+  char* dst = z.ptr[i] + blockIdx.y * z.bs[i] + z.off[i] + e;
+  if ((reinterpret_cast<uintptr_t>(dst) & 15) == 0 && e + 16 <= z.len[i]) {
+    *reinterpret_cast<uint4*>(dst) = make_uint4(0, 0, 0, 0);
+  } else {   // lengths are multiples of 4 bytes
+    for (int j = 0; j < 16 && e + j < z.len[i]; j += 4) *reinterpret_cast<uint32_t*>(dst + j) = 0u;
+  }
+}
+
 __global__ void k_fill_f32(float* p, float v, long long n) {
   const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (e < n) p[e] = v;

@@ -201,11 +201,12 @@ class _LactProgramFn(torch.autograd.Function):
         dw = [torch.empty((b, dh, d), dtype=torch.float32, device=dev),
               torch.empty((b, d, dh), dtype=torch.float32, device=dev),
               torch.empty((b, dh, d), dtype=torch.float32, device=dev)]
-        dq = torch.zeros((b, qa.shape[1], d), dtype=act, device=dev)
-        dk = torch.zeros((b, kv_len, d), dtype=act, device=dev) if has_update else None
-        dv = torch.zeros((b, kv_len, d), dtype=act, device=dev) if has_update else None
-        dlr = [torch.zeros((b, kv_len), dtype=torch.float32, device=dev) if has_update else None for _ in range(3)]
-        dmom = torch.zeros((b, kv_len), dtype=torch.float32, device=dev) if mom is not None else None
+        # lact_backward writes every element of its outputs (rows no step touches are zeroed by the library)
+        dq = torch.empty((b, qa.shape[1], d), dtype=act, device=dev)
+        dk = torch.empty((b, kv_len, d), dtype=act, device=dev) if has_update else None
+        dv = torch.empty((b, kv_len, d), dtype=act, device=dev) if has_update else None
+        dlr = [torch.empty((b, kv_len), dtype=torch.float32, device=dev) if has_update else None for _ in range(3)]
+        dmom = torch.empty((b, kv_len), dtype=torch.float32, device=dev) if mom is not None else None
         stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
         with torch.cuda.device(dev):
             _lib.check(L.lact_backward(ctypes.byref(call.desc), _ptr(qa), _ptr(ka), _ptr(va), _ptr(lr0), _ptr(lr1),
