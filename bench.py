@@ -51,6 +51,9 @@ def main():
     ap.add_argument("--config", default="c1", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-profile", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB device copy (three times): the known-size kernel that scales the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a `rocprofv3 --pmc` run of this command")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures the one-GPU operation only: heads (b = B*H) are independent, so N GPUs would each run "
@@ -76,6 +79,14 @@ def main():
         out = lact_amd.block_causal_lact_swiglu(*[dev[n] for n in order], C, True, dev["momentum"])
         out.backward(go)
         return out
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step()

@@ -103,6 +103,35 @@ __device__ __forceinline__ bf16x8 dma_fetch(const char* tile, int row, int kvec)
   return __builtin_bit_cast(bf16x8, u);
 }
 
+// ---- block -> tile mapping, aware of the 8 accelerator dies (XCDs) ----------------------------------
+// The workgroups of a 1-D grid are dealt to the 8 XCDs round-robin by linear id, and every XCD has its own
+// L2.  Blocks that read the same operands are therefore given ids that are congruent mod 8 and adjacent in
+// that XCD's order, so that the shared tiles are fetched from HBM once and not once per die.  A group is
+// one batch entry with all its tiles (batch count a multiple of 8) or one row of tiles of a batch entry.
+// Only the speed depends on the dealing order, never the result.
+struct TileMap {
+  int gx, gy, gz;   // tiles along x and y, batch entries
+  int by_batch;     // 1: group = batch entry (gx*gy members); 0: group = (batch entry, x tile) (gy members)
+  __host__ __device__ int group_size() const { return by_batch ? gx * gy : gy; }
+  __host__ __device__ int groups() const { return by_batch ? gz : gz * gx; }
+  __host__ __device__ int grid() const { return 8 * ((groups() + 7) / 8) * group_size(); }
+  __device__ __forceinline__ bool locate(int L, int& x, int& y, int& z) const {
+    const int gs = group_size();
+    const int j = L >> 3;
+    const int g = (L & 7) + 8 * (j / gs), m = j % gs;
+    if (g >= groups()) return false;
+    if (by_batch) { z = g; x = m / gy; y = m % gy; }
+    else { z = g / gx; x = g % gx; y = m; }
+    return true;
+  }
+};
+inline TileMap make_tile_map(int gx, int gy, int gz) {
+  TileMap m;
+  m.gx = gx; m.gy = gy; m.gz = gz;
+  m.by_batch = gz % 8 == 0;
+  return m;
+}
+
 // Fragment source of one 32-row MFMA tile: K-contiguous (one ds_read_b128) or K-strided (two transposing reads).
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 template <int ROWS, bool KS>

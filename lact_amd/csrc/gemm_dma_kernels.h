@@ -22,6 +22,7 @@ template <int NT>
 struct RowGemmDmaParams {
   RowGemmParams<NT> g;
   uint16_t* out_ct;   // DUAL: bf16 transposed copy [N][M] (batch stride = bso), or null
+  TileMap map;        // tiles of M, tiles of N, batch
 };
 
 // B_KS: the B operands are [K, N] (N contiguous) instead of [N, K].
@@ -31,7 +32,9 @@ __global__ __launch_bounds__(DMA_THREADS) void k_row_gemm_dma(const RowGemmDmaPa
   constexpr int STAGES = row_stages<TS>();
   using Pipe = DmaPipe<TS, 1, NT, STAGES>;
   const RowGemmParams<NT>& p = pp.g;
-  const int m0 = blockIdx.x * TS::BM, n0 = blockIdx.y * TS::BN, z = blockIdx.z;
+  int bx, by, z;
+  if (!pp.map.locate(blockIdx.x, bx, by, z)) return;
+  const int m0 = bx * TS::BM, n0 = by * TS::BN;
   DmaPhase<1> ph[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
@@ -181,6 +184,7 @@ __global__ __launch_bounds__(DMA_THREADS) void k_row_gemm_dma(const RowGemmDmaPa
 // ------------------------------------------------------------------------------------------------
 struct HiddenDmaParams {
   HiddenParams h;
+  TileMap map;   // token tiles, hidden tiles, batch
 };
 
 template <class TS>
@@ -217,7 +221,9 @@ __global__ __launch_bounds__(DMA_THREADS) void k_apply_hidden_dma(const HiddenDm
   constexpr int STAGES = 3;
   using Pipe = DmaPipe<TS, 2, 1, STAGES>;
   const HiddenParams& p = pp.h;
-  const int m0 = blockIdx.x * TS::BM, n0 = blockIdx.y * TS::BN, z = blockIdx.z;
+  int bx, by, z;
+  if (!pp.map.locate(blockIdx.x, bx, by, z)) return;
+  const int m0 = bx * TS::BM, n0 = by * TS::BN;
   DmaPhase<2> ph[1];
   ph[0].a = token_operand<TS>(p.X, p.bsx, p.ldx, z, m0, p.T);
   ph[0].b[0] = weight_operand(p.W0, p.bsw, p.d, z, n0, p.dh);
@@ -295,7 +301,9 @@ template <class TS>
 __global__ __launch_bounds__(DMA_THREADS) void k_update_hidden_dma(const HiddenDmaParams pp) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const HiddenParams& p = pp.h;
-  const int m0 = blockIdx.x * TS::BM, n0 = blockIdx.y * TS::BN, z = blockIdx.z;
+  int bx, by, z;
+  if (!pp.map.locate(blockIdx.x, bx, by, z)) return;
+  const int m0 = bx * TS::BM, n0 = by * TS::BN;
   f32x16 a02[2][TS::TM][TS::TN], a1[1][TS::TM][TS::TN];
   three_acc_mainloop<TS>(pp, smem, m0, n0, z, a02, a1);
   using SB = StageTile<TS, 2>;
@@ -336,7 +344,9 @@ template <class TS>
 __global__ __launch_bounds__(DMA_THREADS) void k_apply_bwd_hidden_dma(const HiddenDmaParams pp) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const HiddenParams& p = pp.h;
-  const int m0 = blockIdx.x * TS::BM, n0 = blockIdx.y * TS::BN, z = blockIdx.z;
+  int bx, by, z;
+  if (!pp.map.locate(blockIdx.x, bx, by, z)) return;
+  const int m0 = bx * TS::BM, n0 = by * TS::BN;
   f32x16 a02[2][TS::TM][TS::TN], a1[1][TS::TM][TS::TN];
   three_acc_mainloop<TS>(pp, smem, m0, n0, z, a02, a1);
   using SB = StageTile<TS, 2>;
@@ -369,7 +379,9 @@ __global__ __launch_bounds__(DMA_THREADS) void k_update_bwd_hidden_dma(const Hid
   constexpr int STAGES = 3;
   using Pipe = DmaPipe<TS, 2, 3, STAGES>;
   const HiddenParams& p = pp.h;
-  const int m0 = blockIdx.x * TS::BM, n0 = blockIdx.y * TS::BN, z = blockIdx.z;
+  int bx, by, z;
+  if (!pp.map.locate(blockIdx.x, bx, by, z)) return;
+  const int m0 = bx * TS::BM, n0 = by * TS::BN;
   DmaPhase<2> ph[3];
   ph[0].a = token_operand<TS>(p.X, p.bsx, p.ldx, z, m0, p.T);
   ph[0].b[0] = weight_operand(p.W0, p.bsw, p.d, z, n0, p.dh);
@@ -435,9 +447,9 @@ __global__ __launch_bounds__(DMA_THREADS) void k_update_bwd_hidden_dma(const Hid
         SB::put4(lb + 4 * SB::BYTES, tm, tn, g, o4[0], o4[1], o4[2], o4[3]);
         SB::put4(lb + 5 * SB::BYTES, tm, tn, g, o5[0], o5[1], o5[2], o5[3]);
       }
-    store_row_partials<TS>(p, 0, tm, m, z, s0);
-    store_row_partials<TS>(p, 1, tm, m, z, s1);
-    store_row_partials<TS>(p, 2, tm, m, z, s2);
+    store_row_partials<TS>(p, 0, tm, m, z, s0, by);
+    store_row_partials<TS>(p, 1, tm, m, z, s1, by);
+    store_row_partials<TS>(p, 2, tm, m, z, s2, by);
   }
   }
   __syncthreads();
@@ -452,17 +464,22 @@ __global__ __launch_bounds__(DMA_THREADS) void k_update_bwd_hidden_dma(const Hid
 // k_token_reduce_dma: the three token-reduction GEMMs of one step (see k_token_reduce), both operands
 // K-strided (tokens are the rows of every activation), fp32 partials per token split.
 // ------------------------------------------------------------------------------------------------
+struct TokenReduceDmaParams : TokenReduceParams {
+  TileMap map;   // token splits, output tiles, 3 * batch
+};
 template <class TS>
-__global__ __launch_bounds__(DMA_THREADS) void k_token_reduce_dma(const TokenReduceParams p) {
+__global__ __launch_bounds__(DMA_THREADS) void k_token_reduce_dma(const TokenReduceDmaParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int STAGES = row_stages<TS>();
   using Pipe = DmaPipe<TS, 1, 2, STAGES>;
-  const int j = blockIdx.z / p.nb, ib = blockIdx.z % p.nb;
+  int split, tile, bz;   // map: (splits, tiles, 3*nb)
+  if (!p.map.locate(blockIdx.x, split, tile, bz)) return;
+  const int j = bz / p.nb, ib = bz % p.nb;
   const TokenReduceJob& job = p.job[j];
   const int tiles_n = (job.N + TS::BN - 1) / TS::BN;
-  const int m0 = (blockIdx.x / tiles_n) * TS::BM, n0 = (blockIdx.x % tiles_n) * TS::BN;
+  const int m0 = (tile / tiles_n) * TS::BM, n0 = (tile % tiles_n) * TS::BN;
   if (m0 >= job.M) return;
-  const int k_begin = blockIdx.y * p.split_len;
+  const int k_begin = split * p.split_len;
   const int klen = min(p.split_len, p.tokens - k_begin);
   DmaPhase<1> ph[2];
 #pragma unroll
@@ -493,8 +510,8 @@ __global__ __launch_bounds__(DMA_THREADS) void k_token_reduce_dma(const TokenRed
     LACT_FOR_QUADS(TS) ST::put4(lb, tm, tn, g, acc[0][tm][tn][4 * g], acc[0][tm][tn][4 * g + 1], acc[0][tm][tn][4 * g + 2], acc[0][tm][tn][4 * g + 3]);
   }
   __syncthreads();
-  const size_t slot = (size_t)blockIdx.z * p.mat_elems;
-  float* out = p.add_out ? p.add_out + slot : p.partial + (size_t)blockIdx.y * gridDim.z * p.mat_elems + slot;
+  const size_t slot = (size_t)bz * p.mat_elems;
+  float* out = p.add_out ? p.add_out + slot : p.partial + (size_t)split * p.map.gz * p.mat_elems + slot;
   const int r0 = ST::row0(), c0 = ST::col0();
   if (ST::active() && n0 + c0 < job.N) {
     const char* src = smem + (r0 * ST::LD + c0) * 4;

@@ -203,10 +203,10 @@ __global__ __launch_bounds__(TS::THREADS) void k_update_hidden(const HiddenParam
 // Row sums over the hidden dimension of a per-thread partial: lanes l and l^32 hold the same token.
 // Each wave then owns one partial per token; the slot index is (hidden tile, wave column).
 template <class TS>
-__device__ __forceinline__ void store_row_partials(const HiddenParams& p, int which, int tm, int m, int z, float v) {
+__device__ __forceinline__ void store_row_partials(const HiddenParams& p, int which, int tm, int m, int z, float v, int ytile) {
   v += __shfl_xor(v, 32, 64);
   if ((threadIdx.x & 63) < 32 && m < p.T) {
-    const int slot = blockIdx.y * TS::WAVES_N + ((threadIdx.x >> 6) % TS::WAVES_N);
+    const int slot = ytile * TS::WAVES_N + ((threadIdx.x >> 6) % TS::WAVES_N);
     p.lrpart[which * p.lrpart_mat_stride + slot * p.lrpart_stride + (size_t)z * p.Tcap + m] = v;
   }
 }
@@ -319,9 +319,9 @@ __global__ __launch_bounds__(TS::THREADS) void k_update_bwd_hidden(const HiddenP
         Elem<T>::store4(reinterpret_cast<T*>(p.O4) + off, o4[0], o4[1], o4[2], o4[3]);
         Elem<T>::store4(reinterpret_cast<T*>(p.O5) + off, o5[0], o5[1], o5[2], o5[3]);
       }
-    store_row_partials<TS>(p, 0, tm, m, z, s0);
-    store_row_partials<TS>(p, 1, tm, m, z, s1);
-    store_row_partials<TS>(p, 2, tm, m, z, s2);
+    store_row_partials<TS>(p, 0, tm, m, z, s0, blockIdx.y);
+    store_row_partials<TS>(p, 1, tm, m, z, s1, blockIdx.y);
+    store_row_partials<TS>(p, 2, tm, m, z, s2, blockIdx.y);
   }
 }
 

@@ -250,11 +250,12 @@ void launch_row_gemm_dma(const char* site, const RowGemmDmaParams<NT>& q, int ba
   static const std::string name = std::string("k_row_gemm_dma<") + std::to_string(TS::BM) + "x" + std::to_string(TS::BN) + "," +
                                   std::to_string(NT) + (EPI == EPI_STORE ? ",store" : (EPI == EPI_AXPBY ? ",axpby" : ",axpby_dual")) +
                                   (B_KS ? ",Bks>" : ",Bkc>");
-  dim3 grid(ceil_div(q.g.M, TS::BM), ceil_div(q.g.N, TS::BN), batch);
+  RowGemmDmaParams<NT> qq = q;
+  qq.map = make_tile_map(ceil_div(q.g.M, TS::BM), ceil_div(q.g.N, TS::BN), batch);
   double ksum = 0;
   for (int t = 0; t < NT; ++t) ksum += q.g.t[t].K;
-  LACT_LAUNCH_SMEM(name.c_str(), site, 2.0 * q.g.M * q.g.N * ksum * batch, (k_row_gemm_dma<TS, NT, EPI, B_KS>), grid,
-                   dim3(DMA_THREADS), SMEM, s, q);
+  LACT_LAUNCH_SMEM(name.c_str(), site, 2.0 * q.g.M * q.g.N * ksum * batch, (k_row_gemm_dma<TS, NT, EPI, B_KS>), dim3(qq.map.grid()),
+                   dim3(DMA_THREADS), SMEM, s, qq);
 }
 // bf16 with every K a multiple of 64: asynchronous-copy kernels; anything else: the generic tile loop
 template <typename T, bool B_KC, int NT, int EPI>
@@ -394,7 +395,10 @@ struct Runner {
       (void)ver;
       constexpr int SM3 = cmax(DmaSmem<TS_SQ, 2, 3>::BYTES, 3 * StageTile<TS_SQ, 2>::BYTES);
       constexpr int SM6 = cmax(DmaSmem<TS_BWD, 2, 3>::BYTES, 6 * StageTile<TS_BWD, 2>::BYTES);
-      dim3 g3(ceil_div(T_, TS_SQ::BM), ceil_div(d.dh, TS_SQ::BN), d.b), g6(ceil_div(T_, TS_BWD::BM), ceil_div(d.dh, TS_BWD::BN), d.b);
+      const TileMap m3 = make_tile_map(ceil_div(T_, TS_SQ::BM), ceil_div(d.dh, TS_SQ::BN), d.b);
+      const TileMap m6 = make_tile_map(ceil_div(T_, TS_BWD::BM), ceil_div(d.dh, TS_BWD::BN), d.b);
+      q.map = which == 3 ? m6 : m3;
+      dim3 g3(m3.grid()), g6(m6.grid());
       static bool once = (allow_big_lds(k_apply_hidden_dma<TS_SQ>, SM3), allow_big_lds(k_update_hidden_dma<TS_SQ>, SM3),
                           allow_big_lds(k_apply_bwd_hidden_dma<TS_SQ>, SM3), allow_big_lds(k_update_bwd_hidden_dma<TS_BWD>, SM6), true);
       (void)once;
@@ -442,20 +446,23 @@ struct Runner {
         const bool big = d.d % TS_NS::BM == 0 && d.dh % TS_NS::BM == 0;
         const int tiles = big ? (d.d / TS_NS::BM) * (d.dh / TS_NS::BN)
                               : std::max(ceil_div(d.dh, TS_SQ::BM) * ceil_div(d.d, TS_SQ::BN), ceil_div(d.d, TS_SQ::BM) * ceil_div(d.dh, TS_SQ::BN));
-        dim3 g(tiles, sp.n, 3 * d.b);
+        TokenReduceDmaParams pd;
+        static_cast<TokenReduceParams&>(pd) = p;
+        pd.map = make_tile_map(sp.n, tiles, 3 * d.b);
+        dim3 g(pd.map.grid());
         const double fl = 6.0 * tokens * d.d * d.dh * d.b * jobs[0].nterms;
         const bool direct = add_out && sp.n == 1;
-        if (direct) { p.add_out = add_out; p.add_in = coeff != 0.f ? add_in : nullptr; p.coeff = coeff; }
+        if (direct) { pd.add_out = add_out; pd.add_in = coeff != 0.f ? add_in : nullptr; pd.coeff = coeff; }
         if (big) {
           constexpr int SM = cmax(DmaSmem<TS_NS, 1, row_stages<TS_NS>()>::BYTES, StageTile<TS_NS, 4>::BYTES);
           static bool once = (allow_big_lds(k_token_reduce_dma<TS_NS>, SM), true);
           (void)once;
-          LACT_LAUNCH_SMEM("k_token_reduce_dma<192x192>", site, fl, (k_token_reduce_dma<TS_NS>), g, dim3(DMA_THREADS), SM, s, p);
+          LACT_LAUNCH_SMEM("k_token_reduce_dma<192x192>", site, fl, (k_token_reduce_dma<TS_NS>), g, dim3(DMA_THREADS), SM, s, pd);
         } else {
           constexpr int SM = cmax(DmaSmem<TS_SQ, 1, row_stages<TS_SQ>()>::BYTES, StageTile<TS_SQ, 4>::BYTES);
           static bool once = (allow_big_lds(k_token_reduce_dma<TS_SQ>, SM), true);
           (void)once;
-          LACT_LAUNCH_SMEM("k_token_reduce_dma<128x128>", site, fl, (k_token_reduce_dma<TS_SQ>), g, dim3(DMA_THREADS), SM, s, p);
+          LACT_LAUNCH_SMEM("k_token_reduce_dma<128x128>", site, fl, (k_token_reduce_dma<TS_SQ>), g, dim3(DMA_THREADS), SM, s, pd);
         }
         return direct;
       }
