@@ -65,36 +65,41 @@ constexpr int DMA_BK = 64;
 // receives element (i & 3) of the 8 bytes addressed by lanes 4j + (i >> 2), j = 0..3 -- i.e. a 4(k) x 16(r)
 // patch comes back transposed, 4 consecutive k of one r per lane.  The rotation makes the four k-rows of a
 // patch land in different bank groups.
+constexpr int DMA_LOADERS = 2;     // loader waves per block
 template <int ROWS>
 struct DmaLane {
-  static constexpr int N = ROWS / 8;    // copies per K-step
-  static constexpr int G = ROWS / 8;    // granules per k-row of a K-strided tile
+  static constexpr int NALL = ROWS / 8;            // copies per K-step, all loader waves together
+  static constexpr int N = NALL / DMA_LOADERS;     // copies per K-step of this wave: copy lw, lw + DMA_LOADERS, ...
+  static constexpr int G = ROWS / 8;               // granules per k-row of a K-strided tile
+  static_assert(NALL % DMA_LOADERS == 0, "tile rows must split evenly over the loader waves");
   const uint16_t* base;                 // uniform
   size_t kstride;                       // uniform: elements between K-steps
   uint32_t voff[N];                     // byte offset of this lane's granule from base at K-step 0
-  __device__ __forceinline__ void init(const DmaOperand& op) {
+  __device__ __forceinline__ void init(const DmaOperand& op, int lw) {
     const int lane = threadIdx.x & 63;
     base = op.base;
     kstride = op.ks ? (size_t)DMA_BK * op.ld : (size_t)DMA_BK;
 #pragma unroll
-    for (int i = 0; i < N; ++i) {
+    for (int ii = 0; ii < N; ++ii) {
+      const int i = lw + ii * DMA_LOADERS;
       if (op.ks) {
         const int L = i * 64 + lane, k = L / G, p = L % G;
         int g = (p + G - (4 * (k & 3)) % G) % G;
         g = min(g, op.rows / 8 - 1);
-        voff[i] = (uint32_t)(((size_t)k * op.ld + g * 8) * 2);
+        voff[ii] = (uint32_t)(((size_t)k * op.ld + g * 8) * 2);
       } else {
         const int row = i * 8 + (lane >> 3);
         const int kv = ((lane & 7) ^ ((row >> 1) & 7)) * 8;
         const int r = min(row, op.rows - 1);
-        voff[i] = (uint32_t)(((size_t)r * op.ld + kv) * 2);
+        voff[ii] = (uint32_t)(((size_t)r * op.ld + kv) * 2);
       }
     }
   }
+  // lds_tile: LDS address of the tile plus lw * 1024
   __device__ __forceinline__ void issue(int kt, uint32_t lds_tile) const {
     const uint16_t* b = base + kt * kstride;
 #pragma unroll
-    for (int i = 0; i < N; ++i) dma16(b, voff[i], lds_tile + i * 1024);
+    for (int ii = 0; ii < N; ++ii) dma16(b, voff[ii], lds_tile + ii * DMA_LOADERS * 1024);
   }
 };
 
@@ -177,7 +182,7 @@ struct DmaSmem {
   static_assert(BYTES <= 160 * 1024, "ring does not fit the 160 KiB LDS");
 };
 
-constexpr int DMA_THREADS = 320;   // four MFMA waves + one loader wave
+constexpr int DMA_THREADS = 256 + 64 * DMA_LOADERS;   // four MFMA waves + the loader waves
 
 // Flat multi-phase pipeline with a dedicated loader wave.
 //
@@ -201,12 +206,17 @@ struct DmaPipe {
 #pragma unroll
     for (int i = 0; i < NPH; ++i) total += ph[i].K / DMA_BK;
   }
-  __device__ static __forceinline__ bool is_loader() { return __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) == 4; }
+  __device__ static __forceinline__ bool is_loader() { return __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) >= 4; }
 
-  // ---- loader wave: every copy of every phase.  MINLOADS: smallest per-K-step copy count of any phase.
+  // ---- loader waves: every copy of every phase, split evenly.  MINLOADS: smallest per-K-step copy count of
+  // any phase (all loader waves together).  The count of outstanding vector-memory operations of a wave
+  // tops out at 63 -- one wave alone keeps at most 63 KiB in flight, which at 1-2 us of loaded memory
+  // latency caps a compute unit near 40 GB/s; two waves lift that cap above what the ring can hold.
   template <int MINLOADS>
   __device__ __forceinline__ void load_all() {
-    constexpr int AHEAD = (STAGES - 2) * MINLOADS > 63 ? 63 : (STAGES - 2) * MINLOADS;
+    constexpr int PER_WAVE = MINLOADS / DMA_LOADERS;
+    constexpr int AHEAD = (STAGES - 2) * PER_WAVE > 63 ? 63 : (STAGES - 2) * PER_WAVE;
+    const int lw = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) - 4;
     DmaLane<TS::BM> la;
     DmaLane<TS::BN> lb[NBMAX];
     int cp = -1, ckt = 0, cnk = 0, cnb = 0, issued = 0;
@@ -216,15 +226,15 @@ struct DmaPipe {
 #pragma unroll
       for (int i = 0; i < NPH; ++i)
         if (i == cp) {
-          la.init(ph[i].a);
+          la.init(ph[i].a, lw);
 #pragma unroll
-          for (int j = 0; j < NBMAX; ++j) lb[j].init(ph[i].b[j]);
+          for (int j = 0; j < NBMAX; ++j) lb[j].init(ph[i].b[j], lw);
           cnb = ph[i].nb;
           cnk = ph[i].K / DMA_BK;
         }
     };
     auto issue_stage = [&]() {
-      const uint32_t base = lds_addr(smem + (issued % STAGES) * SM::STAGE);
+      const uint32_t base = lds_addr(smem + (issued % STAGES) * SM::STAGE) + lw * 1024;
       la.issue(ckt, base);
 #pragma unroll
       for (int j = 0; j < NBMAX; ++j)
@@ -256,33 +266,44 @@ struct DmaPipe {
     for (int i = 0; i < TS::TM; ++i) sa[i].init((wave / TS::WAVES_N) * TS::WM + i * 32);
 #pragma unroll
     for (int n = 0; n < TS::TN; ++n) sb[n].init((wave % TS::WAVES_N) * TS::WN + n * 32);
-    for (int kt = 0; kt < nk; ++kt, ++step) {
-      __syncthreads();
-      const char* st = smem + (step % STAGES) * SM::STAGE;
-      bf16x8 fa[2][TS::TM], fb[2][NB][TS::TN];
-      auto fetch = [&](int buf, int ks) {
+    if (nk <= 0) return;
+    // Rolling fragment pipeline: the fragments of sub-step s+1 are fetched before the MFMAs of sub-step s
+    // issue, across K-steps too -- the barrier that opens stage kt+1 and the fetch of its first fragments
+    // sit in front of the last MFMA group of stage kt, which hides the LDS latency.
+    bf16x8 fa[2][TS::TM], fb[2][NB][TS::TN];
+    const char* st = nullptr;
+    auto fetch = [&](int buf, int ks) {
 #pragma unroll
-        for (int i = 0; i < TS::TM; ++i) fa[buf][i] = sa[i].fetch(st, ks);
+      for (int i = 0; i < TS::TM; ++i) fa[buf][i] = sa[i].fetch(st, ks);
 #pragma unroll
-        for (int j = 0; j < NB; ++j)
+      for (int j = 0; j < NB; ++j)
 #pragma unroll
-          for (int n = 0; n < TS::TN; ++n) fb[buf][j][n] = sb[n].fetch(st + SM::A_BYTES + j * SM::B_BYTES, ks);
-      };
-      auto mfmas = [&](int buf) {
+        for (int n = 0; n < TS::TN; ++n) fb[buf][j][n] = sb[n].fetch(st + SM::A_BYTES + j * SM::B_BYTES, ks);
+    };
+    auto mfmas = [&](int buf) {
 #pragma unroll
-        for (int j = 0; j < NB; ++j)
+      for (int j = 0; j < NB; ++j)
 #pragma unroll
-          for (int i = 0; i < TS::TM; ++i)
+        for (int i = 0; i < TS::TM; ++i)
 #pragma unroll
-            for (int n = 0; n < TS::TN; ++n) acc[j][i][n] = mma32(fb[buf][j][n], fa[buf][i], acc[j][i][n]);
-      };
-      fetch(0, 0);
+          for (int n = 0; n < TS::TN; ++n) acc[j][i][n] = mma32(fb[buf][j][n], fa[buf][i], acc[j][i][n]);
+    };
+    __syncthreads();
+    st = smem + (step % STAGES) * SM::STAGE;
+    fetch(0, 0);
+    for (int kt = 0; kt < nk; ++kt) {
       fetch(1, 1);
       mfmas(0);
       fetch(0, 2);
       mfmas(1);
       fetch(1, 3);
       mfmas(0);
+      ++step;
+      if (kt + 1 < nk) {
+        __syncthreads();
+        st = smem + (step % STAGES) * SM::STAGE;
+        fetch(0, 0);
+      }
       mfmas(1);
     }
   }
