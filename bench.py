@@ -31,6 +31,21 @@ CONFIGS = {
 }
 
 
+# HBM bytes per launch at config 1 (read + write), from the FETCH_SIZE / WRITE_SIZE counters of two
+# `rocprofv3 --pmc` runs scaled by a 1 GiB copy (profiles/c1_fwd_bwd_hbm_traffic_pmc.txt); MiB.
+MEASURED_TRAFFIC_MIB = {
+    "k_token_reduce_dma<192x192>": 140.5 + 27.0,
+    "k_row_gemm_dma<192x192,2,axpby_dual,Bks>": 81.4 + 40.5,
+    "k_row_gemm_dma<192x192,1,axpby_dual,Bks>": 54.4 + 40.5,
+    "k_row_gemm_dma<192x192,2,axpby,Bkc>": 27.7 + 13.5,
+    "k_row_gemm_dma<192x192,2,store,Bkc>": 27.4 + 13.5,
+    "k_update_bwd_hidden_dma": 130.3 + 148.5,
+    "k_apply_bwd_hidden_dma": 77.9 + 72.0,
+    "k_update_hidden_dma": 78.0 + 72.0,
+    "k_apply_hidden_dma": 33.3 + 24.0,
+}
+
+
 def algorithmic_flops(b, L, d, dh, C, ns_steps=5):
     """Counted FLOPs of fwd+bwd (multiply-add = 2; backward = 2x forward; recompute, momentum, renorm and
     pointwise work not counted): F_apply = 6 d dh T, F_update = 12 d dh T, F_ns = 3 steps (4 r^2 c + 2 r^3)."""
@@ -130,7 +145,10 @@ def main():
         avg_ms = dom["ms"] / dom["launches"]
         achieved = dom["flops"] / dom["launches"] / (avg_ms * 1e-3) / 1e12
         res["roofline"] = {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                           "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None, "kernel": dom_name,
+                           "frac": achieved / PEAK_BF16_TFLOPS,
+                           "traffic": (MEASURED_TRAFFIC_MIB[dom_name] * 2 ** 20
+                                       if args.config == "c1" and dom_name in MEASURED_TRAFFIC_MIB else None),
+                           "kernel": dom_name,
                            "avg_launch_ms": avg_ms, "launches_per_step": dom["launches"] / args.steps,
                            "share_of_kernel_time": dom["ms"] / total_ms}
         res["kernels"] = sorted(
