@@ -131,10 +131,10 @@ struct Plan {
   bool muon = false, bf16 = true, momentum = false;
   size_t mat3 = 0;  // 3*b*elems
   // saved
-  size_t s_wct, s_xbt, s_n0, s_wf, s_wc, s_main, s_d, s_mbar, s_u, s_g16, s_norms, s_xb, s_ab, s_bb, saved_bytes;
+  size_t s_n0, s_wf, s_wc, s_main, s_d, s_mbar, s_u, s_g16, s_norms, s_xb, s_ab, s_bb, saved_bytes;
   // scratch
   size_t t_h[6], t_partial, t_lrpart, t_xf[2], t_xbtmp, t_ss, t_dot, t_mdot, t_gwhat[2], t_gwcur, t_gmcarry, t_gc,
-      t_gxf[2], t_gxb[2], t_sg, t_gas, t_gn0, t_gct, t_gxbt[2], scratch_bytes;
+      t_gxf[2], t_gxb[2], t_sg, t_gas, t_gn0, scratch_bytes;
 
   int build(const lact_desc_t* desc) {
     if (!desc) return fail("null descriptor");
@@ -191,7 +191,6 @@ struct Plan {
     s_n0 = sv.take((size_t)3 * d.b * g.maxrows() * 4);
     s_wf = sv.take((size_t)(nupd + 1) * mat3 * 4);
     s_wc = bf16 ? sv.take((size_t)(nupd + 1) * mat3 * 2) : s_wf;
-    s_wct = bf16 ? sv.take((size_t)(nupd + 1) * mat3 * 2) : 0;
     s_main = d.prenorm ? sv.take((size_t)nupd * mat3 * 4) : 0;
     s_d = sv.take((size_t)nupd * mat3 * 4);
     s_mbar = sv.take((size_t)std::max(1, nupd) * d.b * 4);
@@ -199,7 +198,6 @@ struct Plan {
     s_g16 = muon ? sv.take((size_t)nupd * mat3 * nsz) : 0;
     s_norms = sv.take((size_t)std::max(1, nupd) * 3 * d.b * 4);
     s_xb = muon ? sv.take((size_t)nupd * std::max(1, S) * mat3 * nsz) : 0;
-    s_xbt = (muon && nsz == 2) ? sv.take((size_t)nupd * std::max(1, S) * mat3 * 2) : 0;
     const size_t sq3 = (size_t)3 * d.b * r * r;
     s_ab = muon ? sv.take((size_t)nupd * std::max(1, S) * sq3 * nsz) : 0;
     s_bb = muon ? sv.take((size_t)nupd * std::max(1, S) * sq3 * nsz) : 0;
@@ -223,8 +221,6 @@ struct Plan {
     t_sg = sc.take(sq3 * nsz);
     t_gas = sc.take(sq3 * nsz);
     t_gn0 = sc.take((size_t)3 * d.b * g.maxrows() * 4);
-    t_gct = sc.take(mat3 * 2);
-    for (int i = 0; i < 2; ++i) t_gxbt[i] = sc.take(mat3 * 2);
     scratch_bytes = sc.off + 256;
     return 0;
   }
@@ -359,33 +355,9 @@ struct Runner {
   TN* ab(int u, int it) const { return reinterpret_cast<TN*>(sv + P.s_ab) + ((size_t)u * std::max(1, P.S) + it) * sq3(); }
   TN* bb(int u, int it) const { return reinterpret_cast<TN*>(sv + P.s_bb) + ((size_t)u * std::max(1, P.S) + it) * sq3(); }
   T* h(int i) const { return reinterpret_cast<T*>(sc + P.t_h[i]); }
-  // bf16 activations: transposed bf16 copies of the small matrices feed the asynchronous-copy kernels
   static constexpr bool kBf16 = std::is_same<T, uint16_t>::value;
   static constexpr bool kNsBf16 = std::is_same<TN, uint16_t>::value;
-  uint16_t* wct(int ver) const { return kBf16 ? reinterpret_cast<uint16_t*>(sv + P.s_wct) + (size_t)ver * P.mat3 : nullptr; }
-  uint16_t* wct(int ver, int j) const { return kBf16 ? wct(ver) + (size_t)j * d.b * P.g.elems : nullptr; }
-  uint16_t* xbt(int u, int it) const {
-    return kNsBf16 ? reinterpret_cast<uint16_t*>(sv + P.s_xbt) + ((size_t)u * std::max(1, P.S) + it) * P.mat3 : nullptr;
-  }
-  uint16_t* gct() const { return kBf16 ? reinterpret_cast<uint16_t*>(sc + P.t_gct) : nullptr; }
-  uint16_t* gct(int j) const { return kBf16 ? gct() + (size_t)j * d.b * P.g.elems : nullptr; }
-  uint16_t* gxbt(int i) const { return kNsBf16 ? reinterpret_cast<uint16_t*>(sc + P.t_gxbt[i]) : nullptr; }
 
-  // bf16 transposed copies of packed small matrices (weight orientation or Newton-Schulz orientation)
-  void transpose3(const void* src, uint16_t* dst, bool ns_orientation) const {
-    if (!dst) return;
-    TransposeParams p;
-    p.src = reinterpret_cast<const uint16_t*>(src); p.dst = dst; p.nb = d.b; p.elems = P.g.elems;
-    int mr = 0, mc = 0;
-    for (int j = 0; j < 3; ++j) {
-      p.rows[j] = ns_orientation ? P.r : P.g.rows(j);
-      p.cols[j] = ns_orientation ? P.c : P.g.cols(j);
-      mr = std::max(mr, p.rows[j]); mc = std::max(mc, p.cols[j]);
-    }
-    LACT_LAUNCH("k_transpose_b16", "k_transpose_b16", 0.0, k_transpose_b16, dim3(ceil_div(mc, 64), ceil_div(mr, 64), 3 * d.b), dim3(256), s, p);
-  }
-
-  // the four hidden-layer kernels: asynchronous-copy version for bf16, generic tile loop otherwise
   void launch_hidden(int which, const HiddenParams& hp, int ver, int T_) const {
     const double f = (double)T_ * d.d * d.dh * d.b;
     if (kBf16 && d.d % 64 == 0) {
@@ -495,7 +467,6 @@ struct Runner {
       InitParams p;
       p.g = P.g; p.w[0] = w0; p.w[1] = w1; p.w[2] = w2; p.n0 = n0(); p.wf = wf(0);
       p.wc = P.bf16 ? (void*)wc(0) : nullptr;
-      p.wct = nullptr;
       LACT_LAUNCH("k_init_state", "k_init_state", 0.0, (k_init_state<T>), rowgrid, dim3(256), s, p);
     }
     int ver = 0, u = 0;
@@ -544,6 +515,8 @@ struct Runner {
         p.g16 = P.muon ? g16(u) : nullptr;
         p.ss_part = scr<float>(P.t_ss);
         p.round_partial_bf16 = P.bf16;
+        if (u + 1 == P.nupd && P.momentum && m_out)
+          for (int j = 0; j < 3; ++j) p.m_ext[j] = m_out[j];
         LACT_LAUNCH("k_momentum_prep", "k_momentum_prep", 0.0, (k_momentum_prep<TN>), dim3(P.nblk, 3 * d.b), dim3(256), s, p);
       }
       if (P.muon) {
@@ -551,7 +524,6 @@ struct Runner {
         memset(&p, 0, sizeof(p));
         p.g = P.g; p.g16 = g16(u); p.ss_part = scr<float>(P.t_ss); p.nparts = P.nblk; p.norms = norms(u);
         p.xf = scr<float>(P.t_xf[0]); p.xb = xb(u, 0);
-        p.xbt = nullptr;
         p.u = P.S == 0 ? usave(u) : nullptr;
         p.plain_bf16 = d.ns_mode == LACT_NS_PLAIN_BF16;
         LACT_LAUNCH("k_ns_scale", "k_ns_scale", 0.0, (k_ns_scale<TN>), dim3(P.nblk, 3 * d.b), dim3(256), s, p);
@@ -573,19 +545,20 @@ struct Runner {
         p.main_out = d.prenorm ? main_(u + 1) : nullptr;
         p.wf_out = wf(ver + 1);
         p.wc_out = P.bf16 ? (void*)wc(ver + 1) : nullptr;
-        p.wct_out = nullptr;
+        if (u + 1 == P.nupd && w_out)
+          for (int j = 0; j < 3; ++j) p.w_ext[j] = w_out[j];
         LACT_LAUNCH("k_update_renorm", "k_update_renorm", 0.0, (k_update_renorm<T>), rowgrid, dim3(256), s, p);
       }
       ++ver;
       ++u;
     }
-    const dim3 eg((unsigned)((P.g.elems + 255) / 256), 3 * d.b);
-    if (w_out && (w_out[0] || w_out[1] || w_out[2]))
+    // final weights and momentum state: written by the last update's kernels; copied only when no update ran
+    const dim3 eg((unsigned)((P.g.elems / 4 + 255) / 256), 3 * d.b);
+    if (u == 0 && w_out && (w_out[0] || w_out[1] || w_out[2]))
       LACT_LAUNCH("k_unpack3", "k_unpack3", 0.0, k_unpack3, eg, dim3(256), s, wf(ver), P.g.elems, d.b, w_out[0], w_out[1], w_out[2]);
     if (m_out && (m_out[0] || m_out[1] || m_out[2])) {
-      if (u > 0 && P.momentum)
-        LACT_LAUNCH("k_unpack3", "k_unpack3", 0.0, k_unpack3, eg, dim3(256), s, dsave(u - 1), P.g.elems, d.b, m_out[0], m_out[1], m_out[2]);
-      else
+      if (u > 0 && P.momentum) {
+      } else
         for (int j = 0; j < 3; ++j)
           if (m_out[j]) LACT_LAUNCH("k_fill_f32", "k_fill_f32", 0.0, k_fill_f32, dim3((unsigned)((d.b * P.g.elems + 255) / 256)), dim3(256), s, m_out[j], 0.f, (long long)d.b * P.g.elems);
     }
@@ -651,16 +624,17 @@ struct Runner {
                float* dlr1, float* dlr2, float* dmom) {
     (void)mom;
     const dim3 rowgrid(ceil_div(P.g.maxrows(), 4), 3 * d.b);
-    const dim3 eg((unsigned)((P.g.elems + 255) / 256), 3 * d.b);
-    const dim3 flat((unsigned)((P.mat3 + 255) / 256));
+    const dim3 eg((unsigned)((P.g.elems / 4 + 255) / 256), 3 * d.b);
+    const dim3 flat((unsigned)((P.mat3 / 4 + 255) / 256));
     float* gwcur = scr<float>(P.t_gwcur);
     float* gn0 = scr<float>(P.t_gn0);
     float* gmcarry = scr<float>(P.t_gmcarry);
     float* partial = scr<float>(P.t_partial);
     const long long gn0_n = (long long)3 * d.b * P.g.maxrows();
     LACT_LAUNCH("k_fill_f32", "k_fill_f32", 0.0, k_fill_f32, dim3((unsigned)((gn0_n + 255) / 256)), dim3(256), s, gn0, 0.f, gn0_n);
-    LACT_LAUNCH("k_pack3", "k_pack3", 0.0, k_pack3, eg, dim3(256), s, gwcur, P.g.elems, d.b, dwf ? dwf[0] : nullptr, dwf ? dwf[1] : nullptr,
-                       dwf ? dwf[2] : nullptr);
+    // gwcur: gradient w.r.t. the current weight version; "not valid" stands for zero (nothing written yet)
+    bool gw_valid = dwf && (dwf[0] || dwf[1] || dwf[2]);
+    if (gw_valid) LACT_LAUNCH("k_pack3", "k_pack3", 0.0, k_pack3, eg, dim3(256), s, gwcur, P.g.elems, d.b, dwf[0], dwf[1], dwf[2]);
     // every gradient output is written in full by this call: rows that no step touches are zeroed here
     Touched seen_q, seen_kv;
     {
@@ -706,8 +680,9 @@ struct Runner {
         set_tr_term(jobs[1].t[0], gc, d.do_ld, d.do_bs, h(0), d.dh, hbs());
         jobs[2].M = d.dh; jobs[2].N = d.d;
         set_tr_term(jobs[2].t[0], h(2), d.dh, hbs(), qc, d.q_ld, d.q_bs);
-        if (!token_reduce("apply_bwd_dw", jobs, T_, sp, gwcur, gwcur, 1.f))
-          LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, gwcur, gwcur, 1.f, partial, sp.n, (long long)P.mat3);
+        if (!token_reduce("apply_bwd_dw", jobs, T_, sp, gwcur, gwcur, gw_valid ? 1.f : 0.f))
+          LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, gwcur, gw_valid ? gwcur : nullptr, 1.f, partial, sp.n, (long long)P.mat3);
+        gw_valid = true;
         continue;
       }
       // ---- update u-1: weights ver-1 -> ver
@@ -718,11 +693,11 @@ struct Runner {
       int cur = 0;  // which gxf/gxb buffer holds the running Newton-Schulz gradient
       {
         RenormParams p = renorm_params(u, vprev);
-        p.gy = gwcur;
+        p.gy = gw_valid ? gwcur : nullptr;
         p.carry_in = (d.prenorm && carry_main >= 0) ? scr<float>(P.t_gwhat[carry_main]) : nullptr;
         p.gw_hat = gwhat;
         p.gn0 = gn0;
-        if (P.muon) { p.gxf = scr<float>(P.t_gxf[0]); p.gxb = scr<TN>(P.t_gxb[0]); p.gxbt = nullptr; }
+        if (P.muon) { p.gxf = scr<float>(P.t_gxf[0]); p.gxb = scr<TN>(P.t_gxb[0]); }
         LACT_LAUNCH("k_renorm_bwd", "k_renorm_bwd", 0.0, (k_renorm_bwd<TN>), rowgrid, dim3(256), s, p);
       }
       if (d.prenorm) carry_main = gw_idx;
@@ -777,7 +752,6 @@ struct Runner {
         p.m_prev = (P.momentum && u > 0) ? dsave(u - 1) : nullptr;
         p.mbar = P.momentum ? mbar(u) : nullptr;
         p.gc = scr<T>(P.t_gc);
-        p.gct = nullptr;
         p.mdot_part = scr<float>(P.t_mdot);
         LACT_LAUNCH("k_grad_prep", "k_grad_prep", 0.0, (k_grad_prep<T, TN>), dim3(P.nblk, 3 * d.b), dim3(256), s, p);
         if (P.momentum) {
@@ -832,7 +806,8 @@ struct Runner {
         set_tr_term(jobs[2].t[0], h(2), d.dh, hbs(), kc, d.k_ld, d.k_bs);
         const float pass = d.prenorm ? 0.f : ((P.muon && d.muon_replaces_weight) ? 0.f : 1.f);
         if (!token_reduce("update_bwd_dw", jobs, T_, sp, gwcur, gwhat, pass))
-          LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, gwcur, gwhat, pass, partial, sp.n, (long long)P.mat3);
+          LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, gwcur, pass != 0.f ? gwhat : nullptr, pass, partial, sp.n, (long long)P.mat3);
+        gw_valid = true;
       }
       LACT_LAUNCH("k_lr_reduce", "k_lr_reduce", 0.0, k_lr_reduce, dim3(ceil_div(T_, 256), d.b, 3), dim3(256), s, scr<float>(P.t_lrpart),
                          (long long)P.lr_slots * d.b * P.Tcap, (long long)d.b * P.Tcap,
@@ -842,7 +817,7 @@ struct Runner {
     }
     {
       FinishParams p;
-      p.g = P.g; p.gw = gwcur;
+      p.g = P.g; p.gw = gw_valid ? gwcur : nullptr;
       p.carry = (d.prenorm && carry_main >= 0) ? scr<float>(P.t_gwhat[carry_main]) : nullptr;
       p.gn0 = gn0; p.n0 = n0(); p.w_init = wf(0);
       p.through_norms = d.detach_norms ? 0 : 1;

@@ -17,17 +17,31 @@ struct MatGeom {
   __host__ __device__ int cols(int j) const { return j == 1 ? dh : d; }
   __host__ __device__ bool tall(int j) const { return rows(j) > cols(j); }
   __host__ __device__ int maxrows() const { return d > dh ? d : dh; }
-  // Newton-Schulz orientation is [r, c] = [min, max]; index of the same element in the [c, r] transpose
-  __device__ long long xtidx(long long x) const {
-    const int r = d < dh ? d : dh, c = d < dh ? dh : d;
-    return (x % c) * r + x / c;
-  }
   // index of original element e = i*cols + j inside the Newton-Schulz orientation
   __device__ long long xidx(int j, long long e) const {
     if (!tall(j)) return e;
     const int c = cols(j), r = rows(j);
     const long long i = e / c, k = e % c;
     return k * r + i;
+  }
+};
+
+// All kernels below move 16 bytes per lane wherever an array is walked in its own order (d and dh are
+// multiples of 8, so rows and matrices are multiples of 4 elements); only a matrix that Newton-Schulz holds
+// transposed is addressed element by element.  They are bandwidth-bound: what matters is bytes in flight.
+
+__device__ __forceinline__ float4 ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ void st4(float* p, const float4& v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ float4 f4(float a, float b, float c, float d) { return make_float4(a, b, c, d); }
+__device__ __forceinline__ float dot4(const float4& a, const float4& b) { return a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w; }
+
+// Flat walk of one matrix by the blocks (blockIdx.x) of a (chunks, 3b) grid: [e0, e1), multiples of 4.
+struct FlatRange {
+  long long e0, e1;
+  __device__ __forceinline__ FlatRange(long long elems) {
+    const long long per = ((elems / 4 + gridDim.x - 1) / gridDim.x) * 4;
+    e0 = blockIdx.x * per;
+    e1 = min(e0 + per, elems);
   }
 };
 
@@ -38,7 +52,6 @@ struct InitParams {
   float* n0;              // [3b][maxrows]
   float* wf;              // [3b][elems]
   void* wc;               // [3b][elems] compute type, or null when the compute type is fp32
-  uint16_t* wct;          // [3b][elems] bf16, each matrix transposed ([cols][rows]), or null
 };
 template <typename T>
 __global__ void k_init_state(const InitParams p) {
@@ -47,14 +60,13 @@ __global__ void k_init_state(const InitParams p) {
   if (row >= p.g.rows(j)) return;
   const int cols = p.g.cols(j);
   const float* src = p.w[j] + (size_t)ib * p.g.elems + (size_t)row * cols;
-  float* dst = p.wf + (size_t)z * p.g.elems + (size_t)row * cols;
+  const size_t o = (size_t)z * p.g.elems + (size_t)row * cols;
   float ss = 0.f;
-  for (int c = lane; c < cols; c += 64) {
-    const float v = src[c];
-    ss += v * v;
-    dst[c] = v;
-    if (p.wc) Elem<T>::store(reinterpret_cast<T*>(p.wc) + (size_t)z * p.g.elems + (size_t)row * cols + c, v);
-    if (p.wct) p.wct[(size_t)z * p.g.elems + (size_t)c * p.g.rows(j) + row] = f32_to_bf16(v);
+  for (int c = lane * 4; c < cols; c += 256) {
+    const float4 v = ld4(src + c);
+    ss += dot4(v, v);
+    st4(p.wf + o + c, v);
+    if (p.wc) Elem<T>::store4(reinterpret_cast<T*>(p.wc) + o + c, v.x, v.y, v.z, v.w);
   }
   ss = wave_sum(ss);
   if (lane == 0) p.n0[(size_t)z * p.g.maxrows() + row] = sqrtf(ss);
@@ -77,6 +89,7 @@ struct MomentumPrepParams {
   const float* m_prev;                // [3b][elems] or null (no momentum / first update uses zeros)
   const float* mbar;                  // [b] or null
   float* d_out;                       // [3b][elems]  dw (+ momentum): new momentum state, pre-Muon gradient
+  float* m_ext[3];                    // caller's momentum outputs [b][elems] (same values as d_out), each nullable
   void* g16;                          // [3b][elems]  d_out cast to the Newton-Schulz type, in its orientation, or null
   float* ss_part;                     // [3b][gridDim.x]
   int round_partial_bf16;             // the reduction GEMM's result is a bf16 tensor in the reference
@@ -85,20 +98,35 @@ template <typename TN>
 __global__ void k_momentum_prep(const MomentumPrepParams p) {
   __shared__ float red[16];
   const int z = blockIdx.y, j = z / p.g.nb, ib = z % p.g.nb;
-  const long long per = (p.g.elems + gridDim.x - 1) / gridDim.x;
-  const long long e0 = blockIdx.x * per, e1 = min(e0 + per, p.g.elems);
+  const FlatRange R(p.g.elems);
   const float mb = (p.m_prev && p.mbar) ? p.mbar[ib] : 0.f;
+  const size_t zo = (size_t)z * p.g.elems, stride = (size_t)3 * p.g.nb * p.g.elems;
+  float* ext = p.m_ext[j] ? p.m_ext[j] + (size_t)ib * p.g.elems : nullptr;
+  const bool tall = p.g.tall(j);
   float ss = 0.f;
-  for (long long e = e0 + threadIdx.x; e < e1; e += blockDim.x) {
-    float v = 0.f;
-    for (int s = 0; s < p.nsplit; ++s) v += p.partial[((size_t)s * 3 * p.g.nb + z) * p.g.elems + e];
-    if (p.round_partial_bf16) v = round_bf16(v);
-    if (p.m_prev) v += p.m_prev[(size_t)z * p.g.elems + e] * mb;
-    p.d_out[(size_t)z * p.g.elems + e] = v;
+  for (long long e = R.e0 + threadIdx.x * 4; e < R.e1; e += blockDim.x * 4) {
+    float4 v = ld4(p.partial + zo + e);
+    for (int s = 1; s < p.nsplit; ++s) {
+      const float4 t = ld4(p.partial + s * stride + zo + e);
+      v.x += t.x; v.y += t.y; v.z += t.z; v.w += t.w;
+    }
+    if (p.round_partial_bf16) v = f4(round_bf16(v.x), round_bf16(v.y), round_bf16(v.z), round_bf16(v.w));
+    if (p.m_prev) {
+      const float4 m = ld4(p.m_prev + zo + e);
+      v.x += m.x * mb; v.y += m.y * mb; v.z += m.z * mb; v.w += m.w * mb;
+    }
+    st4(p.d_out + zo + e, v);
+    if (ext) st4(ext + e, v);
     if (p.g16) {
-      const float f = Elem<TN>::rnd(v);
-      Elem<TN>::store(reinterpret_cast<TN*>(p.g16) + (size_t)z * p.g.elems + p.g.xidx(j, e), f);
-      ss += f * f;
+      const float4 f = f4(Elem<TN>::rnd(v.x), Elem<TN>::rnd(v.y), Elem<TN>::rnd(v.z), Elem<TN>::rnd(v.w));
+      TN* g = reinterpret_cast<TN*>(p.g16) + zo;
+      if (!tall) {
+        Elem<TN>::store4(g + e, f.x, f.y, f.z, f.w);
+      } else {
+        Elem<TN>::store(g + p.g.xidx(j, e), f.x); Elem<TN>::store(g + p.g.xidx(j, e + 1), f.y);
+        Elem<TN>::store(g + p.g.xidx(j, e + 2), f.z); Elem<TN>::store(g + p.g.xidx(j, e + 3), f.w);
+      }
+      ss += dot4(f, f);
     }
   }
   if (p.g16) {
@@ -113,7 +141,6 @@ struct NsScaleParams {
   const void* g16; const float* ss_part; int nparts;
   float* norms;          // [3b]
   float* xf; void* xb;   // [3b][elems], Newton-Schulz orientation (fp32 iterate, copy in the Newton-Schulz type)
-  uint16_t* xbt;         // [3b][elems] bf16 copy transposed ([c][r]), or null
   float* u;              // [3b][elems] original orientation, or null (only when zero iterations follow)
   int plain_bf16;        // reference without autocast: norm and quotient are bf16 tensors
 };
@@ -128,16 +155,29 @@ __global__ void k_ns_scale(const NsScaleParams p) {
   float den = n + 1e-7f;
   if (p.plain_bf16) den = round_bf16(den);
   const float inv = 1.f / den;
-  const long long per = (p.g.elems + gridDim.x - 1) / gridDim.x;
-  const long long e0 = blockIdx.x * per, e1 = min(e0 + per, p.g.elems);
-  for (long long e = e0 + threadIdx.x; e < e1; e += blockDim.x) {
-    const long long x = p.g.xidx(j, e);
-    float v = Elem<TN>::load(reinterpret_cast<const TN*>(p.g16) + (size_t)z * p.g.elems + x) * inv;
-    if (p.plain_bf16) v = round_bf16(v);
-    p.xf[(size_t)z * p.g.elems + x] = v;
-    Elem<TN>::store(reinterpret_cast<TN*>(p.xb) + (size_t)z * p.g.elems + x, v);
-    if (p.xbt) p.xbt[(size_t)z * p.g.elems + p.g.xtidx(x)] = f32_to_bf16(v);
-    if (p.u) p.u[(size_t)z * p.g.elems + e] = v;
+  const FlatRange R(p.g.elems);
+  const size_t zo = (size_t)z * p.g.elems;
+  const bool tall = p.g.tall(j);
+  // walks the Newton-Schulz orientation x; the original-orientation copy `u` is the scattered one when tall
+  for (long long x = R.e0 + threadIdx.x * 4; x < R.e1; x += blockDim.x * 4) {
+    float v[4];
+    Elem<TN>::load4(reinterpret_cast<const TN*>(p.g16) + zo + x, v);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[i] *= inv;
+      if (p.plain_bf16) v[i] = round_bf16(v[i]);
+    }
+    st4(p.xf + zo + x, f4(v[0], v[1], v[2], v[3]));
+    Elem<TN>::store4(reinterpret_cast<TN*>(p.xb) + zo + x, v[0], v[1], v[2], v[3]);
+    if (p.u) {
+      if (!tall) {
+        st4(p.u + zo + x, f4(v[0], v[1], v[2], v[3]));
+      } else {   // x = k*rows + i  ->  e = i*cols + k
+        const int rows = p.g.rows(j), cols = p.g.cols(j);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) p.u[zo + (size_t)((x + i) % rows) * cols + (x + i) / rows] = v[i];
+      }
+    }
   }
 }
 
@@ -151,45 +191,68 @@ struct RenormParams {
   int weight_norm;
   float* main_out;                 // un-normalised accumulator (pre-norm) or null
   float* wf_out; void* wc_out;     // new weights: fp32 state and compute-type copy (may be null)
-  uint16_t* wct_out;               // bf16 transposed copy ([cols][rows]) or null
-  uint16_t* gxbt;                  // backward: bf16 transposed copy of the Newton-Schulz-orientation gradient, or null
+  float* w_ext[3];                 // caller's weight outputs [b][elems] (same values as wf_out), each nullable
   // backward only
-  const float* gy;                 // gradient w.r.t. the new weights
+  const float* gy;                 // gradient w.r.t. the new weights, or null (= zero)
   const float* carry_in;           // gradient arriving at the accumulator from later steps (pre-norm) or null
   float* gw_hat;                   // gradient w.r.t. w_hat, original orientation
   float* gn0;                      // [3b][maxrows], accumulated
   float* gxf; void* gxb;           // the same gradient in Newton-Schulz orientation (fp32 + Newton-Schulz type) or null
 };
-__device__ __forceinline__ float renorm_w_hat(const RenormParams& p, size_t off) {
-  float v = p.u[off];
-  if (p.cw != 0.f) v += p.cw * p.base[off];
-  if (p.raw) v += p.cr * p.raw[off];
+__device__ __forceinline__ float4 renorm_w_hat4(const RenormParams& p, size_t off) {
+  float4 v = ld4(p.u + off);
+  if (p.cw != 0.f) {
+    const float4 b = ld4(p.base + off);
+    v.x += p.cw * b.x; v.y += p.cw * b.y; v.z += p.cw * b.z; v.w += p.cw * b.w;
+  }
+  if (p.raw) {
+    const float4 r = ld4(p.raw + off);
+    v.x += p.cr * r.x; v.y += p.cr * r.y; v.z += p.cr * r.z; v.w += p.cr * r.w;
+  }
   return v;
 }
+constexpr int ROW_VEC_MAX = 4;   // a lane keeps up to 4 x 4 elements of its row in registers (rows up to 1024 columns)
 template <typename T>
 __global__ void k_update_renorm(const RenormParams p) {
-  const int z = blockIdx.y, j = z / p.g.nb;
+  const int z = blockIdx.y, j = z / p.g.nb, ib = z % p.g.nb;
   const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (row >= p.g.rows(j)) return;
   const int cols = p.g.cols(j);
   const size_t o = (size_t)z * p.g.elems + (size_t)row * cols;
+  float* ext = p.w_ext[j] ? p.w_ext[j] + (size_t)ib * p.g.elems + (size_t)row * cols : nullptr;
+  const bool keep = cols <= 256 * ROW_VEC_MAX;
+  float4 vv[ROW_VEC_MAX];
   float ss = 0.f;
-  for (int c = lane; c < cols; c += 64) {
-    const float v = renorm_w_hat(p, o + c);
-    ss += v * v;
+#pragma unroll
+  for (int i = 0; i < ROW_VEC_MAX; ++i) {
+    const int c = lane * 4 + i * 256;
+    if (c < cols) {
+      vv[i] = renorm_w_hat4(p, o + c);
+      ss += dot4(vv[i], vv[i]);
+    }
+  }
+  for (int c = lane * 4 + ROW_VEC_MAX * 256; c < cols; c += 256) {
+    const float4 v = renorm_w_hat4(p, o + c);
+    ss += dot4(v, v);
   }
   ss = wave_sum(ss);
   const float den = sqrtf(ss) + 1e-5f;
   const float n0 = p.weight_norm ? p.n0[(size_t)z * p.g.maxrows() + row] : 1.f;
-  for (int c = lane; c < cols; c += 64) {
-    const float v = renorm_w_hat(p, o + c);
-    if (p.main_out) p.main_out[o + c] = v;
+  auto emit = [&](int c, const float4& v) {
+    if (p.main_out) st4(p.main_out + o + c, v);
     // same operation order as the reference: (w / (norm + eps)) * w_norm
-    const float y = p.weight_norm ? (v / den) * n0 : v;
-    p.wf_out[o + c] = y;
-    if (p.wc_out) Elem<T>::store(reinterpret_cast<T*>(p.wc_out) + o + c, y);
-    if (p.wct_out) p.wct_out[(size_t)z * p.g.elems + (size_t)c * p.g.rows(j) + row] = f32_to_bf16(y);
+    const float4 y = p.weight_norm ? f4((v.x / den) * n0, (v.y / den) * n0, (v.z / den) * n0, (v.w / den) * n0) : v;
+    st4(p.wf_out + o + c, y);
+    if (ext) st4(ext + c, y);
+    if (p.wc_out) Elem<T>::store4(reinterpret_cast<T*>(p.wc_out) + o + c, y.x, y.y, y.z, y.w);
+  };
+#pragma unroll
+  for (int i = 0; i < ROW_VEC_MAX; ++i) {
+    const int c = lane * 4 + i * 256;
+    if (c < cols) emit(c, vv[i]);
   }
+  if (!keep)
+    for (int c = lane * 4 + ROW_VEC_MAX * 256; c < cols; c += 256) emit(c, renorm_w_hat4(p, o + c));
 }
 
 // backward of the line above.  y = w_hat*n0/(r+eps), r = ||w_hat||:
@@ -199,15 +262,16 @@ __global__ void k_renorm_bwd(const RenormParams p) {
   const int z = blockIdx.y, j = z / p.g.nb;
   const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (row >= p.g.rows(j)) return;
-  const int cols = p.g.cols(j);
-  const size_t o = (size_t)z * p.g.elems + (size_t)row * cols;
+  const int cols = p.g.cols(j), rows = p.g.rows(j);
+  const size_t zo = (size_t)z * p.g.elems, o = zo + (size_t)row * cols;
+  const bool tall = p.g.tall(j);
   float c0 = 1.f, c1 = 0.f;
   if (p.weight_norm) {
     float ss = 0.f, dot = 0.f;
-    for (int c = lane; c < cols; c += 64) {
-      const float v = renorm_w_hat(p, o + c);
-      ss += v * v;
-      dot += v * p.gy[o + c];
+    for (int c = lane * 4; c < cols; c += 256) {
+      const float4 v = renorm_w_hat4(p, o + c);
+      ss += dot4(v, v);
+      if (p.gy) dot += dot4(v, ld4(p.gy + o + c));
     }
     ss = wave_sum(ss);
     dot = wave_sum(dot);
@@ -216,16 +280,31 @@ __global__ void k_renorm_bwd(const RenormParams p) {
     c1 = r > 0.f ? dot * n0 / (r * (r + 1e-5f) * (r + 1e-5f)) : 0.f;
     if (lane == 0) p.gn0[(size_t)z * p.g.maxrows() + row] += dot / (r + 1e-5f);
   }
-  for (int c = lane; c < cols; c += 64) {
-    float gv = p.gy[o + c] * c0;
-    if (p.weight_norm) gv -= renorm_w_hat(p, o + c) * c1;
-    if (p.carry_in) gv += p.carry_in[o + c];
-    p.gw_hat[o + c] = gv;
+  for (int c = lane * 4; c < cols; c += 256) {
+    float4 gv = p.gy ? ld4(p.gy + o + c) : f4(0.f, 0.f, 0.f, 0.f);
+    gv = f4(gv.x * c0, gv.y * c0, gv.z * c0, gv.w * c0);
+    if (p.weight_norm) {
+      const float4 w = renorm_w_hat4(p, o + c);
+      gv.x -= w.x * c1; gv.y -= w.y * c1; gv.z -= w.z * c1; gv.w -= w.w * c1;
+    }
+    if (p.carry_in) {
+      const float4 ci = ld4(p.carry_in + o + c);
+      gv.x += ci.x; gv.y += ci.y; gv.z += ci.z; gv.w += ci.w;
+    }
+    st4(p.gw_hat + o + c, gv);
     if (p.gxf) {
-      const size_t x = (size_t)z * p.g.elems + p.g.xidx(j, (long long)row * cols + c);
-      p.gxf[x] = gv;
-      Elem<TN>::store(reinterpret_cast<TN*>(p.gxb) + x, gv);
-      if (p.gxbt) p.gxbt[(size_t)z * p.g.elems + p.g.xtidx(x - (size_t)z * p.g.elems)] = f32_to_bf16(gv);
+      if (!tall) {
+        st4(p.gxf + o + c, gv);
+        Elem<TN>::store4(reinterpret_cast<TN*>(p.gxb) + o + c, gv.x, gv.y, gv.z, gv.w);
+      } else {   // element (row, c) sits at c*rows + row in the Newton-Schulz orientation
+        const float g[4] = {gv.x, gv.y, gv.z, gv.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const size_t x = zo + (size_t)(c + i) * rows + row;
+          p.gxf[x] = g[i];
+          Elem<TN>::store(reinterpret_cast<TN*>(p.gxb) + x, g[i]);
+        }
+      }
     }
   }
 }
@@ -239,11 +318,14 @@ template <typename TN>
 __global__ void k_ns_bwd_dot(const NsDotParams p) {
   __shared__ float red[16];
   const int z = blockIdx.y;
-  const long long per = (p.g.elems + gridDim.x - 1) / gridDim.x;
-  const long long e0 = blockIdx.x * per, e1 = min(e0 + per, p.g.elems);
+  const FlatRange R(p.g.elems);
+  const size_t zo = (size_t)z * p.g.elems;
   float s = 0.f;
-  for (long long e = e0 + threadIdx.x; e < e1; e += blockDim.x)
-    s += p.gx0[(size_t)z * p.g.elems + e] * Elem<TN>::load(reinterpret_cast<const TN*>(p.g16) + (size_t)z * p.g.elems + e);
+  for (long long e = R.e0 + threadIdx.x * 4; e < R.e1; e += blockDim.x * 4) {
+    float g[4];
+    Elem<TN>::load4(reinterpret_cast<const TN*>(p.g16) + zo + e, g);
+    s += dot4(ld4(p.gx0 + zo + e), f4(g[0], g[1], g[2], g[3]));
+  }
   s = block_sum(s, red);
   if (threadIdx.x == 0) p.dot_part[(size_t)z * gridDim.x + blockIdx.x] = s;
 }
@@ -256,7 +338,6 @@ struct GradPrepParams {
   float* gm_carry; int carry_valid;  // gradient w.r.t. the momentum state after this update (in/out)
   const float* m_prev; const float* mbar;   // null without momentum
   void* gc;                          // [3b][elems] compute-type copy of d loss / d dw  (GEMM operand)
-  uint16_t* gct;                     // bf16 transposed copy ([cols][rows]) or null
   float* mdot_part;                  // [3b][gridDim.x] partial <g, m_prev>
 };
 template <typename T, typename TN>
@@ -272,29 +353,46 @@ __global__ void k_grad_prep(const GradPrepParams p) {
     c1 = n > 0.f ? dot / (n * (n + 1e-7f) * (n + 1e-7f)) : 0.f;
   }
   const float mb = p.mbar ? p.mbar[ib] : 0.f;
-  const long long per = (p.g.elems + gridDim.x - 1) / gridDim.x;
-  const long long e0 = blockIdx.x * per, e1 = min(e0 + per, p.g.elems);
+  const FlatRange R(p.g.elems);
+  const size_t zo = (size_t)z * p.g.elems;
+  const bool tall = p.g.tall(j);
   float md = 0.f;
-  for (long long e = e0 + threadIdx.x; e < e1; e += blockDim.x) {
-    const size_t o = (size_t)z * p.g.elems + e;
-    float gv;
+  for (long long e = R.e0 + threadIdx.x * 4; e < R.e1; e += blockDim.x * 4) {
+    const size_t o = zo + e;
+    float4 gv;
     if (p.muon) {
-      const size_t x = (size_t)z * p.g.elems + p.g.xidx(j, e);
-      gv = p.gx0[x] * c0 - Elem<TN>::load(reinterpret_cast<const TN*>(p.g16) + x) * c1;
-      if (p.cr != 0.f) gv += p.cr * p.gw_hat[o];
+      float4 gx;
+      float g[4];
+      if (!tall) {
+        gx = ld4(p.gx0 + o);
+        Elem<TN>::load4(reinterpret_cast<const TN*>(p.g16) + o, g);
+      } else {
+        float t[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const size_t x = zo + p.g.xidx(j, e + i);
+          t[i] = p.gx0[x];
+          g[i] = Elem<TN>::load(reinterpret_cast<const TN*>(p.g16) + x);
+        }
+        gx = f4(t[0], t[1], t[2], t[3]);
+      }
+      gv = f4(gx.x * c0 - g[0] * c1, gx.y * c0 - g[1] * c1, gx.z * c0 - g[2] * c1, gx.w * c0 - g[3] * c1);
+      if (p.cr != 0.f) {
+        const float4 w = ld4(p.gw_hat + o);
+        gv.x += p.cr * w.x; gv.y += p.cr * w.y; gv.z += p.cr * w.z; gv.w += p.cr * w.w;
+      }
     } else {
-      gv = p.gw_hat[o];
+      gv = ld4(p.gw_hat + o);
     }
     if (p.gm_carry) {
-      if (p.carry_valid) gv += p.gm_carry[o];
-      p.gm_carry[o] = gv * mb;                       // d/d M_prev of  dw + M_prev * mbar
-      if (p.m_prev) md += gv * p.m_prev[o];
+      if (p.carry_valid) {
+        const float4 cv = ld4(p.gm_carry + o);
+        gv.x += cv.x; gv.y += cv.y; gv.z += cv.z; gv.w += cv.w;
+      }
+      st4(p.gm_carry + o, f4(gv.x * mb, gv.y * mb, gv.z * mb, gv.w * mb));   // d/d M_prev of  dw + M_prev * mbar
+      if (p.m_prev) md += dot4(gv, ld4(p.m_prev + o));
     }
-    Elem<T>::store(reinterpret_cast<T*>(p.gc) + o, gv);
-    if (p.gct) {
-      const int cols = p.g.cols(j);
-      p.gct[(size_t)z * p.g.elems + (e % cols) * p.g.rows(j) + e / cols] = f32_to_bf16(gv);
-    }
+    Elem<T>::store4(reinterpret_cast<T*>(p.gc) + o, gv.x, gv.y, gv.z, gv.w);
   }
   if (p.gm_carry) {
     md = block_sum(md, red);
@@ -312,13 +410,20 @@ __global__ void k_momentum_grad(const float* mdot_part, int nparts, int nb, floa
   for (int t = threadIdx.x; t < len; t += blockDim.x) dmom[ib * bs + start + t] += s;
 }
 
-// out = coeff*in_add + sum of split partials
+// out = coeff*in_add + sum of split partials; 4 elements per thread (total is a multiple of 4)
 __global__ void k_reduce_partials(float* out, const float* in_add, float coeff, const float* partial, int nsplit, long long total) {
-  const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long e = ((long long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (e >= total) return;
-  float v = in_add ? coeff * in_add[e] : 0.f;
-  for (int s = 0; s < nsplit; ++s) v += partial[(size_t)s * total + e];
-  out[e] = v;
+  float4 v = f4(0.f, 0.f, 0.f, 0.f);
+  if (in_add) {
+    const float4 a = ld4(in_add + e);
+    v = f4(coeff * a.x, coeff * a.y, coeff * a.z, coeff * a.w);
+  }
+  for (int s = 0; s < nsplit; ++s) {
+    const float4 t = ld4(partial + (size_t)s * total + e);
+    v.x += t.x; v.y += t.y; v.z += t.z; v.w += t.w;
+  }
+  st4(out + e, v);
 }
 
 // dlr_j[ib, start + t] += sum over slots of the row partials
@@ -351,62 +456,34 @@ __global__ void k_finish_weight_grads(const FinishParams p) {
     c = n > 0.f ? p.gn0[(size_t)z * p.g.maxrows() + row] / n : 0.f;
   }
   float* dst = p.out[j] + (size_t)ib * p.g.elems + (size_t)row * cols;
-  for (int k = lane; k < cols; k += 64) {
-    float v = p.gw[o + k];
-    if (p.carry) v += p.carry[o + k];
-    if (p.through_norms) v += c * p.w_init[o + k];
-    dst[k] = v;
+  for (int k = lane * 4; k < cols; k += 256) {
+    float4 v = p.gw ? ld4(p.gw + o + k) : f4(0.f, 0.f, 0.f, 0.f);
+    if (p.carry) {
+      const float4 t = ld4(p.carry + o + k);
+      v.x += t.x; v.y += t.y; v.z += t.z; v.w += t.w;
+    }
+    if (p.through_norms) {
+      const float4 w = ld4(p.w_init + o + k);
+      v.x += c * w.x; v.y += c * w.y; v.z += c * w.z; v.w += c * w.w;
+    }
+    st4(dst + k, v);
   }
 }
 
-// unpack [3b][elems] into the three caller tensors
+// [3b][elems] <-> the three caller tensors, 4 elements per thread
 __global__ void k_unpack3(const float* src, long long elems, int nb, float* o0, float* o1, float* o2) {
-  const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long e = ((long long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   const int z = blockIdx.y;
   if (e >= elems) return;
   float* dst = (z / nb) == 0 ? o0 : ((z / nb) == 1 ? o1 : o2);
-  if (dst) dst[(size_t)(z % nb) * elems + e] = src[(size_t)z * elems + e];
+  if (dst) st4(dst + (size_t)(z % nb) * elems + e, ld4(src + (size_t)z * elems + e));
 }
 __global__ void k_pack3(float* dst, long long elems, int nb, const float* i0, const float* i1, const float* i2) {
-  const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long e = ((long long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   const int z = blockIdx.y;
   if (e >= elems) return;
   const float* src = (z / nb) == 0 ? i0 : ((z / nb) == 1 ? i1 : i2);
-  dst[(size_t)z * elems + e] = src ? src[(size_t)(z % nb) * elems + e] : 0.f;
-}
-// dst[z][c*rows + r] = src[z][r*cols + c] for bf16 matrices; kind j = z / nb picks (rows, cols).
-struct TransposeParams {
-  const uint16_t* src; uint16_t* dst;
-  int rows[3], cols[3];
-  int nb; long long elems;
-};
-__global__ __launch_bounds__(256) void k_transpose_b16(const TransposeParams p) {
-  __shared__ uint16_t tile[64][66];
-  const int z = blockIdx.z, j = z / p.nb;
-  const int rows = p.rows[j], cols = p.cols[j];
-  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
-  if (r0 >= rows || c0 >= cols) return;
-  const uint16_t* src = p.src + (size_t)z * p.elems;
-  uint16_t* dst = p.dst + (size_t)z * p.elems;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int idx = threadIdx.x + i * 256, r = idx / 16, c = (idx % 16) * 4;
-    uint2 v = make_uint2(0, 0);
-    if (r0 + r < rows && c0 + c < cols) v = *reinterpret_cast<const uint2*>(src + (size_t)(r0 + r) * cols + c0 + c);
-    tile[r][c] = (uint16_t)(v.x & 0xffff); tile[r][c + 1] = (uint16_t)(v.x >> 16);
-    tile[r][c + 2] = (uint16_t)(v.y & 0xffff); tile[r][c + 3] = (uint16_t)(v.y >> 16);
-  }
-  __syncthreads();
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int idx = threadIdx.x + i * 256, c = idx / 16, r = (idx % 16) * 4;
-    if (c0 + c < cols && r0 + r < rows) {
-      uint2 v;
-      v.x = (uint32_t)tile[r][c] | ((uint32_t)tile[r + 1][c] << 16);
-      v.y = (uint32_t)tile[r + 2][c] | ((uint32_t)tile[r + 3][c] << 16);
-      *reinterpret_cast<uint2*>(dst + (size_t)(c0 + c) * rows + r0 + r) = v;
-    }
-  }
+  st4(dst + (size_t)z * elems + e, src ? ld4(src + (size_t)(z % nb) * elems + e) : f4(0.f, 0.f, 0.f, 0.f));
 }
 
 // Zero up to 16 strided byte ranges in one launch: segment i covers, for every batch ib < nb, the bytes

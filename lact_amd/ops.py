@@ -173,6 +173,7 @@ class _LactProgramFn(torch.autograd.Function):
         ctx.mom_dtype = momentum.dtype if momentum is not None else None
         ctx.save_for_backward(qa, ka, va, lrs[0], lrs[1], lrs[2], mom, saved)
         ctx.mark_non_differentiable(*[m for m in m_out if m is not None])
+        ctx.set_materialize_grads(False)   # unused outputs arrive as None in backward, not as zero tensors
         out_dtype = q.dtype if q.dtype in (torch.bfloat16, torch.float32) else act
         if v is not None and v.dtype == torch.float32 and act == torch.bfloat16:
             out_dtype = torch.float32          # zeros_like(v) receives the bf16 products
