@@ -8,6 +8,7 @@
 #include <cstring>
 #include <string>
 #include <vector>
+#include <mutex>
 
 #include <type_traits>
 
@@ -97,6 +98,36 @@ template <> const char* tname<float>() { return "f32"; }
     if (e_ != hipSuccess) return fail(std::string("kernel launch failed: ") + hipGetErrorString(e_)); \
   } while (0)
 
+// ---- side stream: the apply steps of a program do not depend on the update chain that runs beside them
+// (block-causal: apply(i) and update(i) both read weight version i), so they are enqueued on a second
+// stream of default priority, forked from and joined back into the caller's stream with events.  The
+// memory-bound tails of one chain then overlap the matrix work of the other.  One stream and one event
+// pool per device, created on first use and kept until the process ends.
+struct SideCtx {
+  hipStream_t stream = nullptr;
+  std::vector<hipEvent_t> ev;
+  size_t next = 0;
+  hipEvent_t event() {
+    if (next == ev.size()) {
+      hipEvent_t e;
+      (void)hipEventCreateWithFlags(&e, hipEventDisableTiming);
+      ev.push_back(e);
+    }
+    return ev[next++];
+  }
+};
+bool g_overlap = true;
+std::mutex g_enqueue_mutex;   // one program is enqueued at a time (the side-stream context is shared)
+SideCtx* side_ctx() {
+  static SideCtx ctx[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+  SideCtx& c = ctx[dev];
+  if (!c.stream && hipStreamCreateWithFlags(&c.stream, hipStreamNonBlocking) != hipSuccess) return nullptr;
+  c.next = 0;
+  return &c;
+}
+
 using TSA = TileShape<128, 128, 2, 2>;  // two or three accumulators
 using TSB = TileShape<64, 128, 2, 2>;   // six accumulators (update backward)
 
@@ -134,7 +165,7 @@ struct Plan {
   size_t s_n0, s_wf, s_wc, s_main, s_d, s_mbar, s_u, s_g16, s_norms, s_xb, s_ab, s_bb, saved_bytes;
   // scratch
   size_t t_h[6], t_partial, t_lrpart, t_xf[2], t_xbtmp, t_ss, t_dot, t_mdot, t_gwhat[2], t_gwcur, t_gmcarry, t_gc,
-      t_gxf[2], t_gxb[2], t_sg, t_gas, t_gn0, scratch_bytes;
+      t_gxf[2], t_gxb[2], t_sg, t_gas, t_gn0, t_hs[3], t_partial_side, t_gwside[2], scratch_bytes;
 
   int build(const lact_desc_t* desc) {
     if (!desc) return fail("null descriptor");
@@ -221,6 +252,10 @@ struct Plan {
     t_sg = sc.take(sq3 * nsz);
     t_gas = sc.take(sq3 * nsz);
     t_gn0 = sc.take((size_t)3 * d.b * g.maxrows() * 4);
+    // the apply steps' own buffers (they run beside the update chain)
+    for (int i = 0; i < 3; ++i) t_hs[i] = sc.take((size_t)d.b * Tcap * d.dh * esz);
+    t_partial_side = sc.take((size_t)nsplit_max * mat3 * 4);
+    for (int i = 0; i < 2; ++i) t_gwside[i] = sc.take(mat3 * 4);
     scratch_bytes = sc.off + 256;
     return 0;
   }
@@ -336,8 +371,28 @@ struct Runner {
   char* sv;   // saved
   char* sc;   // scratch
   const lact_desc_t& d;
+  hipStream_t s_main, s_side;   // caller's stream; stream of the apply steps (= s_main when overlap is off)
+  SideCtx* side = nullptr;
+  const size_t* hsel;           // token-major intermediates of the chain being enqueued
+  size_t partial_sel;
   Runner(const Plan& p, void* saved, void* scratch, hipStream_t st)
-      : P(p), s(st), sv(align256(saved)), sc(align256(scratch)), d(p.d) {}
+      : P(p), s(st), sv(align256(saved)), sc(align256(scratch)), d(p.d), s_main(st), s_side(st), hsel(p.t_h), partial_sel(p.t_partial) {
+    if (g_overlap) side = side_ctx();
+    if (side) s_side = side->stream;
+  }
+  // `waiter` waits for everything enqueued so far on `on`
+  void wait_for(hipStream_t waiter, hipStream_t on) {
+    if (waiter == on || !side) return;
+    hipEvent_t e = side->event();
+    (void)hipEventRecord(e, on);
+    (void)hipStreamWaitEvent(waiter, e, 0);
+  }
+  // enqueue on the side chain (its stream and buffers) while this object lives
+  struct OnSide {
+    Runner& r;
+    explicit OnSide(Runner& rr) : r(rr) { r.s = r.s_side; r.hsel = r.P.t_hs; r.partial_sel = r.P.t_partial_side; }
+    ~OnSide() { r.s = r.s_main; r.hsel = r.P.t_h; r.partial_sel = r.P.t_partial; }
+  };
 
   float* n0() const { return reinterpret_cast<float*>(sv + P.s_n0); }
   float* wf(int ver) const { return reinterpret_cast<float*>(sv + P.s_wf) + (size_t)ver * P.mat3; }
@@ -354,7 +409,7 @@ struct Runner {
   size_t sq3() const { return (size_t)3 * d.b * P.r * P.r; }
   TN* ab(int u, int it) const { return reinterpret_cast<TN*>(sv + P.s_ab) + ((size_t)u * std::max(1, P.S) + it) * sq3(); }
   TN* bb(int u, int it) const { return reinterpret_cast<TN*>(sv + P.s_bb) + ((size_t)u * std::max(1, P.S) + it) * sq3(); }
-  T* h(int i) const { return reinterpret_cast<T*>(sc + P.t_h[i]); }
+  T* h(int i) const { return reinterpret_cast<T*>(sc + hsel[i]); }
   static constexpr bool kBf16 = std::is_same<T, uint16_t>::value;
   static constexpr bool kNsBf16 = std::is_same<TN, uint16_t>::value;
 
@@ -412,7 +467,7 @@ struct Runner {
     memset(&p, 0, sizeof(p));
     for (int i = 0; i < 3; ++i) p.job[i] = jobs[i];
     p.nb = d.b; p.tokens = tokens; p.split_len = sp.len;
-    p.partial = scr<float>(P.t_partial); p.mat_elems = P.g.elems;
+    p.partial = scr<float>(partial_sel); p.mat_elems = P.g.elems;
     if constexpr (kBf16) {
       if (sp.len % 64 == 0 && tokens % 64 == 0 && d.d % 8 == 0 && d.dh % 8 == 0) {
         const bool big = d.d % TS_NS::BM == 0 && d.dh % TS_NS::BM == 0;
@@ -470,9 +525,17 @@ struct Runner {
       LACT_LAUNCH("k_init_state", "k_init_state", 0.0, (k_init_state<T>), rowgrid, dim3(256), s, p);
     }
     int ver = 0, u = 0;
+    int side_has_ver = -1;     // newest weight version the side stream has been made to wait for
+    bool side_used = false;
     for (const auto& st : P.steps) {
       const int T_ = st.end - st.start;
       if (st.kind == LACT_APPLY) {
+        if (side_has_ver < ver) {
+          wait_for(s_side, s_main);
+          side_has_ver = ver;
+        }
+        side_used = true;
+        OnSide on_side(*this);
         HiddenParams hp = hidden_params(T_, q + (size_t)st.start * d.q_ld, d.q_ld, d.q_bs, nullptr, 0, 0, ver);
         hp.O0 = h(0);
         launch_hidden(0, hp, ver, T_);
@@ -552,6 +615,7 @@ struct Runner {
       ++ver;
       ++u;
     }
+    if (side_used) wait_for(s_main, s_side);
     // final weights and momentum state: written by the last update's kernels; copied only when no update ran
     const dim3 eg((unsigned)((P.g.elems / 4 + 255) / 256), 3 * d.b);
     if (u == 0 && w_out && (w_out[0] || w_out[1] || w_out[2]))
@@ -650,6 +714,15 @@ struct Runner {
       for (float* ptr : small) zl.add(ptr, (long long)d.kv_len * 4, 0, (long long)d.kv_len * 4);
       zl.flush();
     }
+    // The apply steps run on the side stream.  Their weight gradients go to gw_side[version & 1] and are added
+    // by the consumer of that version's gradient (the renorm backward of the update that made the version, or
+    // the final kernel); `free_ev` orders the reuse of a gw_side buffer after its consumer.
+    wait_for(s_side, s_main);
+    float* gw_side[2] = {scr<float>(P.t_gwside[0]), scr<float>(P.t_gwside[1])};
+    bool side_valid[2] = {false, false};
+    hipEvent_t free_ev[2] = {nullptr, nullptr};
+    bool side_used = false;
+    float* partial_side = scr<float>(P.t_partial_side);
     int ver = P.nupd, u = P.nupd;
     int carry_main = -1;       // index of the gwhat buffer holding the accumulator's gradient (pre-norm)
     bool gm_valid = false;     // gmcarry holds d loss / d (momentum state after update u-1)
@@ -658,6 +731,13 @@ struct Runner {
       const int T_ = st.end - st.start;
       const Split sp = choose_split(T_, P.tiles * 3 * d.b);
       if (st.kind == LACT_APPLY) {
+        const int sb = ver & 1;
+        if (!side_valid[sb] && free_ev[sb] && s_side != s_main) {
+          (void)hipStreamWaitEvent(s_side, free_ev[sb], 0);
+          free_ev[sb] = nullptr;
+        }
+        side_used = true;
+        OnSide on_side(*this);
         const T* qc = q + (size_t)st.start * d.q_ld;
         const T* gc = dout + (size_t)st.out_start * d.do_ld;
         HiddenParams hp = hidden_params(T_, qc, d.q_ld, d.q_bs, gc, d.do_ld, d.do_bs, ver);
@@ -680,9 +760,9 @@ struct Runner {
         set_tr_term(jobs[1].t[0], gc, d.do_ld, d.do_bs, h(0), d.dh, hbs());
         jobs[2].M = d.dh; jobs[2].N = d.d;
         set_tr_term(jobs[2].t[0], h(2), d.dh, hbs(), qc, d.q_ld, d.q_bs);
-        if (!token_reduce("apply_bwd_dw", jobs, T_, sp, gwcur, gwcur, gw_valid ? 1.f : 0.f))
-          LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, gwcur, gw_valid ? gwcur : nullptr, 1.f, partial, sp.n, (long long)P.mat3);
-        gw_valid = true;
+        if (!token_reduce("apply_bwd_dw", jobs, T_, sp, gw_side[sb], gw_side[sb], side_valid[sb] ? 1.f : 0.f))
+          LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, gw_side[sb], side_valid[sb] ? gw_side[sb] : nullptr, 1.f, partial_side, sp.n, (long long)P.mat3);
+        side_valid[sb] = true;
         continue;
       }
       // ---- update u-1: weights ver-1 -> ver
@@ -694,11 +774,23 @@ struct Runner {
       {
         RenormParams p = renorm_params(u, vprev);
         p.gy = gw_valid ? gwcur : nullptr;
+        const int sb = ver & 1;
+        if (side_valid[sb]) {
+          wait_for(s_main, s_side);
+          p.gy2 = gw_side[sb];
+        }
         p.carry_in = (d.prenorm && carry_main >= 0) ? scr<float>(P.t_gwhat[carry_main]) : nullptr;
         p.gw_hat = gwhat;
         p.gn0 = gn0;
         if (P.muon) { p.gxf = scr<float>(P.t_gxf[0]); p.gxb = scr<TN>(P.t_gxb[0]); }
         LACT_LAUNCH("k_renorm_bwd", "k_renorm_bwd", 0.0, (k_renorm_bwd<TN>), rowgrid, dim3(256), s, p);
+        if (side_valid[sb]) {
+          side_valid[sb] = false;
+          if (side) {
+            free_ev[sb] = side->event();
+            (void)hipEventRecord(free_ev[sb], s_main);
+          }
+        }
       }
       if (d.prenorm) carry_main = gw_idx;
       if (P.muon) {
@@ -817,7 +909,9 @@ struct Runner {
     }
     {
       FinishParams p;
+      if (side_used) wait_for(s_main, s_side);
       p.g = P.g; p.gw = gw_valid ? gwcur : nullptr;
+      p.gw2 = side_valid[0] ? gw_side[0] : nullptr;
       p.carry = (d.prenorm && carry_main >= 0) ? scr<float>(P.t_gwhat[carry_main]) : nullptr;
       p.gn0 = gn0; p.n0 = n0(); p.w_init = wf(0);
       p.through_norms = d.detach_norms ? 0 : 1;
@@ -903,6 +997,13 @@ extern "C" {
 const char* lact_last_error(void) { return g_err.c_str(); }
 int lact_version(void) { return 1; }
 
+int lact_set_stream_overlap(int on) {
+  std::lock_guard<std::mutex> lock(g_enqueue_mutex);
+  const int was = g_overlap ? 1 : 0;
+  g_overlap = on != 0;
+  return was;
+}
+
 int lact_profile_enable(int on) {
   g_prof.clear();
   g_prof.on = on != 0;
@@ -960,6 +1061,7 @@ int lact_forward(const lact_desc_t* desc, const float* w0, const float* w1, cons
   if (P.nupd > 0 && check_ptrs({k, v, lr0, lr1, lr2}, "k, v, lr")) return -1;
   if (P.nupd > 0 && P.momentum && !momentum) return fail("use_momentum set but momentum is null");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  std::lock_guard<std::mutex> lock(g_enqueue_mutex);
 #define LACT_FWD(T_, TN_)                                                                                           \
   {                                                                                                                 \
     Runner<T_, TN_> R(P, saved, scratch, s);                                                                        \
@@ -986,6 +1088,7 @@ int lact_backward(const lact_desc_t* desc, const void* q, const void* k, const v
   const int al = P.bf16 ? 8 : 4;
   if (P.d.do_ld % al || P.d.do_bs % al || P.d.do_ld < P.d.d) return fail("dout strides must keep 16-byte alignment");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  std::lock_guard<std::mutex> lock(g_enqueue_mutex);
 #define LACT_BWD(T_, TN_)                                                                                            \
   {                                                                                                                  \
     Runner<T_, TN_> R(P, const_cast<void*>(saved), scratch, s);                                                      \

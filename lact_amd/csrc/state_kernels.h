@@ -194,6 +194,7 @@ struct RenormParams {
   float* w_ext[3];                 // caller's weight outputs [b][elems] (same values as wf_out), each nullable
   // backward only
   const float* gy;                 // gradient w.r.t. the new weights, or null (= zero)
+  const float* gy2;                // second addend of the same gradient (the apply steps' share), or null
   const float* carry_in;           // gradient arriving at the accumulator from later steps (pre-norm) or null
   float* gw_hat;                   // gradient w.r.t. w_hat, original orientation
   float* gn0;                      // [3b][maxrows], accumulated
@@ -210,6 +211,14 @@ __device__ __forceinline__ float4 renorm_w_hat4(const RenormParams& p, size_t of
     v.x += p.cr * r.x; v.y += p.cr * r.y; v.z += p.cr * r.z; v.w += p.cr * r.w;
   }
   return v;
+}
+__device__ __forceinline__ float4 renorm_gy4(const RenormParams& p, size_t off) {
+  float4 g = p.gy ? ld4(p.gy + off) : f4(0.f, 0.f, 0.f, 0.f);
+  if (p.gy2) {
+    const float4 t = ld4(p.gy2 + off);
+    g.x += t.x; g.y += t.y; g.z += t.z; g.w += t.w;
+  }
+  return g;
 }
 constexpr int ROW_VEC_MAX = 4;   // a lane keeps up to 4 x 4 elements of its row in registers (rows up to 1024 columns)
 template <typename T>
@@ -271,7 +280,7 @@ __global__ void k_renorm_bwd(const RenormParams p) {
     for (int c = lane * 4; c < cols; c += 256) {
       const float4 v = renorm_w_hat4(p, o + c);
       ss += dot4(v, v);
-      if (p.gy) dot += dot4(v, ld4(p.gy + o + c));
+      if (p.gy || p.gy2) dot += dot4(v, renorm_gy4(p, o + c));
     }
     ss = wave_sum(ss);
     dot = wave_sum(dot);
@@ -281,7 +290,7 @@ __global__ void k_renorm_bwd(const RenormParams p) {
     if (lane == 0) p.gn0[(size_t)z * p.g.maxrows() + row] += dot / (r + 1e-5f);
   }
   for (int c = lane * 4; c < cols; c += 256) {
-    float4 gv = p.gy ? ld4(p.gy + o + c) : f4(0.f, 0.f, 0.f, 0.f);
+    float4 gv = renorm_gy4(p, o + c);
     gv = f4(gv.x * c0, gv.y * c0, gv.z * c0, gv.w * c0);
     if (p.weight_norm) {
       const float4 w = renorm_w_hat4(p, o + c);
@@ -440,7 +449,7 @@ __global__ void k_lr_reduce(const float* lrpart, long long mat_stride, long long
 // final weight gradients: state gradient (+ accumulator carry) + the path through the initial row norms
 struct FinishParams {
   MatGeom g;
-  const float* gw; const float* carry; const float* gn0; const float* n0; const float* w_init;
+  const float* gw; const float* gw2; const float* carry; const float* gn0; const float* n0; const float* w_init;   // gw, gw2: addends, nullable
   int through_norms;
   float* out[3];
 };
@@ -458,6 +467,10 @@ __global__ void k_finish_weight_grads(const FinishParams p) {
   float* dst = p.out[j] + (size_t)ib * p.g.elems + (size_t)row * cols;
   for (int k = lane * 4; k < cols; k += 256) {
     float4 v = p.gw ? ld4(p.gw + o + k) : f4(0.f, 0.f, 0.f, 0.f);
+    if (p.gw2) {
+      const float4 t = ld4(p.gw2 + o + k);
+      v.x += t.x; v.y += t.y; v.z += t.z; v.w += t.w;
+    }
     if (p.carry) {
       const float4 t = ld4(p.carry + o + k);
       v.x += t.x; v.y += t.y; v.z += t.z; v.w += t.w;

@@ -438,3 +438,39 @@ def test_config1_full_size_properties():
     assert torch.equal(out4, out1[perm]) and torch.equal(gr4["w1"], gr1["w1"][perm]) and torch.equal(gr4["k"], gr1["k"][perm])
     # with momentum == 0 after the only update nothing is carried: d loss / d momentum is <g, M_prev> = 0
     assert float(gr1["momentum"].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("prenorm", [False, True])
+def test_stream_overlap_is_bit_identical(prenorm):
+    """The apply steps run on the library's second stream beside the update chain (forked and joined with
+    events).  With the overlap switched off everything is enqueued on the caller's stream: both must give the
+    same bits, over several chunks (the apply steps' weight-gradient buffers alternate by weight version)
+    and over back-to-back calls."""
+    say("stream overlap on/off, prenorm", prenorm)
+    from lact_amd import _lib
+    b, L, d, dh, C = 4, 5 * 256, 128, 128, 256
+    inp = problem(b, L, d, dh, seed=77, act=torch.bfloat16)
+    go = torch.randn(b, L, d, generator=torch.Generator().manual_seed(5)).bfloat16().to(DEV)
+    fn = T.prenorm_block_causal_lact_swiglu if prenorm else T.block_causal_lact_swiglu
+
+    def run():
+        res = []
+        for _ in range(3):                       # back-to-back: the second stream's work of one call meets the next
+            t = clone_to(inp, DEV)
+            out = fn(*args9(t), C, True, t["momentum"])
+            res.append((out, grads_of(out, t, go)))
+        torch.cuda.synchronize()
+        return res
+    L_ = _lib.lib()
+    prev = L_.lact_set_stream_overlap(1)
+    try:
+        on = run()
+        L_.lact_set_stream_overlap(0)
+        off = run()
+    finally:
+        L_.lact_set_stream_overlap(prev)
+    for (o1, g1), (o0, g0) in zip(on, off):
+        assert torch.equal(o1, o0)
+        for n in g0:
+            assert torch.equal(g1[n], g0[n]), n
+    assert torch.equal(on[0][0], on[2][0]) and all(torch.equal(on[0][1][n], on[2][1][n]) for n in on[0][1])
