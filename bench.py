@@ -67,7 +67,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-profile", action="store_true")
     ap.add_argument("--no-overlap", action="store_true",
-                    help="keep the apply steps on the caller's stream (lact_set_stream_overlap(0)): kernels then run "
+                    help="keep the apply steps on the caller's stream (LACT_OPT_STREAM_OVERLAP off): kernels then run "
                          "one at a time and their durations are those of the kernel alone; used for profiles")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (three times): the known-size kernel that scales the "
@@ -107,7 +107,7 @@ def main():
         del src, dst
 
     if args.no_overlap:
-        _lib.lib().lact_set_stream_overlap(0)
+        _lib.lib().lact_set_option(_lib.OPT_STREAM_OVERLAP, 0)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -134,14 +134,14 @@ def main():
     #      the kernels run on (a second pass, so that the events do not perturb `value`)
     if not args.no_kernel_profile:
         Lb = _lib.lib()
-        Lb.lact_set_stream_overlap(0)      # one kernel at a time: the duration of a launch is that kernel's own
+        Lb.lact_set_option(_lib.OPT_STREAM_OVERLAP, 0)      # one kernel at a time: the duration of a launch is that kernel's own
         Lb.lact_profile_enable(1)
         for _ in range(args.steps):
             step()
         buf = ctypes.create_string_buffer(1 << 20)
         _lib.check(Lb.lact_profile_report(buf, len(buf)))
         Lb.lact_profile_enable(0)
-        Lb.lact_set_stream_overlap(0 if args.no_overlap else 1)
+        Lb.lact_set_option(_lib.OPT_STREAM_OVERLAP, 0 if args.no_overlap else 1)
         rows = json.loads(buf.value.decode())
         by_kernel = {}
         for r in rows:

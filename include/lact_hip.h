@@ -102,13 +102,18 @@ size_t lact_newton_schulz_workspace_bytes(int32_t n, int32_t rows, int32_t cols,
 int lact_newton_schulz(int32_t n, int32_t rows, int32_t cols, const float* g, float* out, int32_t steps,
                        const float* coeffs, int32_t ns_mode, void* workspace, void* stream);
 
-/* The apply steps of a program are independent of the update chain that runs beside them; by default
- * lact_forward / lact_backward enqueue them on a library-owned second stream (default priority, one per
- * device, created on first use) that is forked from and joined back into the caller's stream with events,
- * so the call stays asynchronous and ordered on the caller's stream as a whole.  on = 0 keeps everything
- * on the caller's stream.  Returns the previous setting.  No counterpart in the reference (PyTorch
- * enqueues the whole layer on one stream). */
-int lact_set_stream_overlap(int on);
+/* Execution options (process-wide; no counterpart in the reference, where PyTorch enqueues the whole layer on one
+ * stream as separate kernels).  Both are on by default and change no result bit.
+ *   LACT_OPT_STREAM_OVERLAP: the apply steps of a program do not depend on the update chain that runs beside
+ *     them; lact_forward / lact_backward enqueue them on a library-owned second stream (default priority, one
+ *     per device, created on first use) that is forked from and joined back into the caller's stream with
+ *     events, so the call as a whole stays asynchronous and ordered on the caller's stream.
+ *   LACT_OPT_FUSED_NEWTON_SCHULZ: all Newton-Schulz iterations of an update (and of its backward) run as one
+ *     kernel whose blocks meet at per-matrix barriers (bf16, rows and columns multiples of 192, at most 8
+ *     iterations); otherwise three GEMM launches per iteration.
+ * Returns the previous value (0 / 1), or -1 for an unknown option. */
+enum { LACT_OPT_STREAM_OVERLAP = 0, LACT_OPT_FUSED_NEWTON_SCHULZ = 1 };
+int lact_set_option(int32_t option, int32_t value);
 
 /* Per-launch timing with HIP events on the caller's stream (no counterpart in the reference, which
  * times with wall-clock prints, lact_ar_video/minVid/train.py:458-460).  While enabled every kernel

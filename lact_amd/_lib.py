@@ -32,8 +32,9 @@ class Desc(Structure):
     ]
 
 
+OPT_STREAM_OVERLAP, OPT_FUSED_NEWTON_SCHULZ = 0, 1
 EXPORTS = ("lact_last_error", "lact_version", "lact_query_sizes", "lact_forward", "lact_backward",
-           "lact_newton_schulz_workspace_bytes", "lact_newton_schulz", "lact_set_stream_overlap", "lact_profile_enable",
+           "lact_newton_schulz_workspace_bytes", "lact_newton_schulz", "lact_set_option", "lact_profile_enable",
            "lact_profile_report")
 
 _lib = None
@@ -61,8 +62,8 @@ def lib():
     L.lact_newton_schulz_workspace_bytes.restype = c_size_t
     L.lact_newton_schulz.argtypes = [c_int32, c_int32, c_int32, vp, vp, c_int32, POINTER(c_float), c_int32, vp, vp]
     L.lact_newton_schulz.restype = c_int32
-    L.lact_set_stream_overlap.argtypes = [c_int32]
-    L.lact_set_stream_overlap.restype = c_int32
+    L.lact_set_option.argtypes = [c_int32, c_int32]
+    L.lact_set_option.restype = c_int32
     L.lact_profile_enable.argtypes = [c_int32]
     L.lact_profile_enable.restype = c_int32
     L.lact_profile_report.argtypes = [c_char_p, c_size_t]

@@ -28,9 +28,19 @@ __device__ __forceinline__ uint32_t lds_addr(const void* p) {
 
 // 16 bytes per lane from global memory (uniform 64-bit base + per-lane 32-bit byte offset) to LDS: lane i
 // lands at lds_base + 16*i (lds_base wave-uniform).  No vector-ALU work per copy: bases live in SGPRs.
+// SC1: device-scope load -- always misses the vector L1 and is served by the L2.  Used where the data was written
+// by another compute unit during this same kernel (the L1 is not coherent with other units' stores).
+template <bool SC1 = false>
 __device__ __forceinline__ void dma16(const void* sbase, uint32_t voff, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t" ::"s"(lds_base), "v"(voff), "s"(sbase)
-               : "memory", "m0");
+#ifdef LACT_EXP_NO_DMA
+  return;
+#endif
+  if (SC1)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 sc1\n\t" ::"s"(lds_base), "v"(voff), "s"(sbase)
+                 : "memory", "m0");
+  else
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t" ::"s"(lds_base), "v"(voff), "s"(sbase)
+                 : "memory", "m0");
 }
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
@@ -96,10 +106,11 @@ struct DmaLane {
     }
   }
   // lds_tile: LDS address of the tile plus lw * 1024
+  template <bool SC1>
   __device__ __forceinline__ void issue(int kt, uint32_t lds_tile) const {
     const uint16_t* b = base + kt * kstride;
 #pragma unroll
-    for (int ii = 0; ii < N; ++ii) dma16(b, voff[ii], lds_tile + ii * DMA_LOADERS * 1024);
+    for (int ii = 0; ii < N; ++ii) dma16<SC1>(b, voff[ii], lds_tile + ii * DMA_LOADERS * 1024);
   }
 };
 
@@ -174,6 +185,18 @@ struct FragSrc {
   }
 };
 
+// Scheduling directive: MFMAS matrix instructions with READS LDS reads spread behind the first of them.
+template <int READS, int MFMAS, int I = 0>
+__device__ __forceinline__ void sched_interleave() {
+  if constexpr (I < MFMAS) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    constexpr int RPM = (READS + MFMAS - 1) / MFMAS;
+    constexpr int left = READS - I * RPM;
+    if constexpr (left > 0) __builtin_amdgcn_sched_group_barrier(0x100, left < RPM ? left : RPM, 0);
+    sched_interleave<READS, MFMAS, I + 1>();
+  }
+}
+
 template <class TS, int NBMAX, int STAGES>
 struct DmaSmem {
   static constexpr int A_BYTES = TS::BM * 128, B_BYTES = TS::BN * 128;
@@ -193,7 +216,7 @@ constexpr int DMA_THREADS = 256 + 64 * DMA_LOADERS;   // four MFMA waves + the l
 // only read fragments and issue MFMAs.  One barrier per K-step:
 //     loader:    wait until stage kt has landed; barrier; refill the stage the MFMA waves just left
 //     consumers: barrier; MFMAs on stage kt
-template <class TS, int NBMAX, int NPH, int STAGES>
+template <class TS, int NBMAX, int NPH, int STAGES, bool SC1 = false>
 struct DmaPipe {
   using SM = DmaSmem<TS, NBMAX, STAGES>;
   static constexpr int loads(int nb) { return (TS::BM + nb * TS::BN) / 8; }   // loader copies per K-step
@@ -235,10 +258,10 @@ struct DmaPipe {
     };
     auto issue_stage = [&]() {
       const uint32_t base = lds_addr(smem + (issued % STAGES) * SM::STAGE) + lw * 1024;
-      la.issue(ckt, base);
+      la.template issue<SC1>(ckt, base);
 #pragma unroll
       for (int j = 0; j < NBMAX; ++j)
-        if (j < cnb) lb[j].issue(ckt, base + SM::A_BYTES + j * SM::B_BYTES);
+        if (j < cnb) lb[j].template issue<SC1>(ckt, base + SM::A_BYTES + j * SM::B_BYTES);
       ++issued;
       if (++ckt == cnk)
         while (cp + 1 < NPH) {
@@ -288,16 +311,27 @@ struct DmaPipe {
 #pragma unroll
           for (int n = 0; n < TS::TN; ++n) acc[j][i][n] = mma32(fb[buf][j][n], fa[buf][i], acc[j][i][n]);
     };
+    // Instruction order within a (fetch next, MFMAs current) pair: LDS reads behind each of the first MFMAs,
+    // so that the reads spread under the matrix work instead of piling up in front of a wait.
+    constexpr int READS = (A_KS ? 2 : 1) * TS::TM + (B_KS ? 2 : 1) * NB * TS::TN, MFMAS = NB * TS::TM * TS::TN;
+    auto interleave = [&]() {
+#ifndef LACT_EXP_NO_SCHED
+      sched_interleave<READS, MFMAS>();
+#endif
+    };
     __syncthreads();
     st = smem + (step % STAGES) * SM::STAGE;
     fetch(0, 0);
     for (int kt = 0; kt < nk; ++kt) {
       fetch(1, 1);
       mfmas(0);
+      interleave();
       fetch(0, 2);
       mfmas(1);
+      interleave();
       fetch(1, 3);
       mfmas(0);
+      interleave();
       ++step;
       if (kt + 1 < nk) {
         __syncthreads();
@@ -305,6 +339,7 @@ struct DmaPipe {
         fetch(0, 0);
       }
       mfmas(1);
+      interleave();
     }
   }
 };

@@ -25,15 +25,16 @@ struct RowGemmDmaParams {
   TileMap map;        // tiles of M, tiles of N, batch
 };
 
-// B_KS: the B operands are [K, N] (N contiguous) instead of [N, K].
-template <class TS, int NT, int EPI, bool B_KS>
-__global__ __launch_bounds__(DMA_THREADS) void k_row_gemm_dma(const RowGemmDmaParams<NT> pp) {
-  extern __shared__ __attribute__((aligned(16))) char smem[];
+// One output tile (bx, by) of batch entry z.  B_KS: the B operands are [K, N] (N contiguous) instead of [N, K].
+// SC1: the operands were written by other compute units during this kernel (loads bypass the vector L1); the
+// auxiliary tile of the blending epilogues is always one this block wrote itself or an earlier kernel wrote.
+// All threads of the block must call it; on return the LDS may still be read by this block's epilogue, so the
+// caller synchronises the block before the LDS is written again.
+template <class TS, int NT, int EPI, bool B_KS, bool SC1>
+__device__ __forceinline__ void row_gemm_tile(const RowGemmDmaParams<NT>& pp, int bx, int by, int z, char* smem) {
   constexpr int STAGES = row_stages<TS>();
-  using Pipe = DmaPipe<TS, 1, NT, STAGES>;
+  using Pipe = DmaPipe<TS, 1, NT, STAGES, SC1>;
   const RowGemmParams<NT>& p = pp.g;
-  int bx, by, z;
-  if (!pp.map.locate(blockIdx.x, bx, by, z)) return;
   const int m0 = bx * TS::BM, n0 = by * TS::BN;
   DmaPhase<1> ph[NT];
 #pragma unroll
@@ -177,6 +178,14 @@ __global__ __launch_bounds__(DMA_THREADS) void k_row_gemm_dma(const RowGemmDmaPa
     }
   }
   LACT_TS(3);
+}
+
+template <class TS, int NT, int EPI, bool B_KS>
+__global__ __launch_bounds__(DMA_THREADS) void k_row_gemm_dma(const RowGemmDmaParams<NT> pp) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  int bx, by, z;
+  if (!pp.map.locate(blockIdx.x, bx, by, z)) return;
+  row_gemm_tile<TS, NT, EPI, B_KS, false>(pp, bx, by, z, smem);
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -13,6 +13,7 @@
 #include <type_traits>
 
 #include "gemm_dma_kernels.h"
+#include "ns_fused.h"
 #include "gemm_kernels.h"
 #include "state_kernels.h"
 
@@ -107,6 +108,8 @@ struct SideCtx {
   hipStream_t stream = nullptr;
   std::vector<hipEvent_t> ev;
   size_t next = 0;
+  hipEvent_t fused_done = nullptr;   // completion of the newest fused Newton-Schulz kernel of this process
+  bool fused_recorded = false;
   hipEvent_t event() {
     if (next == ev.size()) {
       hipEvent_t e;
@@ -117,6 +120,7 @@ struct SideCtx {
   }
 };
 bool g_overlap = true;
+bool g_fused_ns = true;
 std::mutex g_enqueue_mutex;   // one program is enqueued at a time (the side-stream context is shared)
 SideCtx* side_ctx() {
   static SideCtx ctx[64];
@@ -165,7 +169,7 @@ struct Plan {
   size_t s_n0, s_wf, s_wc, s_main, s_d, s_mbar, s_u, s_g16, s_norms, s_xb, s_ab, s_bb, saved_bytes;
   // scratch
   size_t t_h[6], t_partial, t_lrpart, t_xf[2], t_xbtmp, t_ss, t_dot, t_mdot, t_gwhat[2], t_gwcur, t_gmcarry, t_gc,
-      t_gxf[2], t_gxb[2], t_sg, t_gas, t_gn0, t_hs[3], t_partial_side, t_gwside[2], scratch_bytes;
+      t_gxf[2], t_gxb[2], t_sg, t_gas, t_gn0, t_hs[3], t_partial_side, t_gwside[2], t_nssync, scratch_bytes;
 
   int build(const lact_desc_t* desc) {
     if (!desc) return fail("null descriptor");
@@ -256,6 +260,7 @@ struct Plan {
     for (int i = 0; i < 3; ++i) t_hs[i] = sc.take((size_t)d.b * Tcap * d.dh * esz);
     t_partial_side = sc.take((size_t)nsplit_max * mat3 * 4);
     for (int i = 0; i < 2; ++i) t_gwside[i] = sc.take(mat3 * 4);
+    t_nssync = sc.take(((size_t)3 * d.b * 32 + 32) * 4);   // per-matrix barrier lines of the fused Newton-Schulz kernel + error word
     scratch_bytes = sc.off + 256;
     return 0;
   }
@@ -377,8 +382,40 @@ struct Runner {
   size_t partial_sel;
   Runner(const Plan& p, void* saved, void* scratch, hipStream_t st)
       : P(p), s(st), sv(align256(saved)), sc(align256(scratch)), d(p.d), s_main(st), s_side(st), hsel(p.t_h), partial_sel(p.t_partial) {
-    if (g_overlap) side = side_ctx();
-    if (side) s_side = side->stream;
+    side = side_ctx();
+    if (side && g_overlap) s_side = side->stream;
+  }
+  // ---- fused Newton-Schulz: one launch per batch of at most 256 resident blocks
+  bool ns_fused_ok() const {
+    if (!g_fused_ns || !side || !kNsBf16 || P.S < 1 || P.S > NS_FUSED_MAX_STEPS) return false;
+    if (P.r % TS_NS::BM || P.c % TS_NS::BN) return false;
+    return (P.r / TS_NS::BM) * (P.c / TS_NS::BN) <= 32;
+  }
+  template <bool BWD>
+  void launch_ns_fused(NsFusedParams p) {
+    constexpr int SM = cmax(DmaSmem<TS_NS, 1, row_stages<TS_NS>()>::BYTES, StageTile<TS_NS, 4>::BYTES);
+    static bool once = (allow_big_lds(k_ns_fused<BWD>, SM), true);
+    (void)once;
+    const int total = 3 * d.b, nbm = (P.r / TS_NS::BM) * (P.c / TS_NS::BN);
+    const int per = (256 / nbm) / 8 * 8;
+    unsigned* sync = scr<unsigned>(P.t_nssync);
+    const long long words = (long long)total * 32 + 32;
+    LACT_LAUNCH("k_fill_f32", "k_fill_f32", 0.0, k_fill_f32, dim3((unsigned)((words + 255) / 256)), dim3(256), s, reinterpret_cast<float*>(sync), 0.f, words);
+    p.r = P.r; p.c = P.c; p.S = P.S; p.nb = d.b; p.mask = tall_mask();
+    for (int i = 0; i < 3 * P.S; ++i) p.coeffs[i] = P.coeffs[i];
+    p.error = sync + (size_t)total * 32;
+    const double terms = BWD ? 6.0 : 3.0;
+    for (int z0 = 0; z0 < total; z0 += per) {
+      p.z0 = z0; p.n = std::min(per, total - z0); p.sync = sync + (size_t)z0 * 32;
+      const int grid = 8 * ((p.n + 7) / 8) * nbm;
+      // fused launches of this process never overlap each other (each needs its groups resident as a whole)
+      if (side->fused_recorded) (void)hipStreamWaitEvent(s, side->fused_done, 0);
+      LACT_LAUNCH_SMEM(BWD ? "k_ns_fused<bwd>" : "k_ns_fused<fwd>", BWD ? "ns_bwd" : "ns_fwd", terms * 2.0 * P.r * P.r * P.c * P.S * p.n,
+                       (k_ns_fused<BWD>), dim3(grid), dim3(DMA_THREADS), SM, s, p);
+      if (!side->fused_done) (void)hipEventCreateWithFlags(&side->fused_done, hipEventDisableTiming);
+      (void)hipEventRecord(side->fused_done, s);
+      side->fused_recorded = true;
+    }
   }
   // `waiter` waits for everything enqueued so far on `on`
   void wait_for(hipStream_t waiter, hipStream_t on) {
@@ -590,6 +627,18 @@ struct Runner {
         p.u = P.S == 0 ? usave(u) : nullptr;
         p.plain_bf16 = d.ns_mode == LACT_NS_PLAIN_BF16;
         LACT_LAUNCH("k_ns_scale", "k_ns_scale", 0.0, (k_ns_scale<TN>), dim3(P.nblk, 3 * d.b), dim3(256), s, p);
+        if (ns_fused_ok()) {
+          if constexpr (kNsBf16) {
+            NsFusedParams f;
+            memset(&f, 0, sizeof(f));
+            f.plain = d.ns_mode == LACT_NS_PLAIN_BF16;
+            f.xf[0] = scr<float>(P.t_xf[0]); f.xf[1] = scr<float>(P.t_xf[1]);
+            f.xb = xb(u, 0); f.xb_it_stride = (long long)P.mat3;
+            f.ab = ab(u, 0); f.bb = bb(u, 0); f.sq_it_stride = (long long)sq3();
+            f.xb_last = scr<uint16_t>(P.t_xbtmp); f.u_out = usave(u);
+            launch_ns_fused<false>(f);
+          }
+        } else
         for (int it = 0; it < P.S; ++it) {
           const bool last = it + 1 == P.S;
           NsIter I;
@@ -610,6 +659,7 @@ struct Runner {
         p.wc_out = P.bf16 ? (void*)wc(ver + 1) : nullptr;
         if (u + 1 == P.nupd && w_out)
           for (int j = 0; j < 3; ++j) p.w_ext[j] = w_out[j];
+        if (P.muon && ns_fused_ok()) p.poison = scr<unsigned>(P.t_nssync) + (size_t)3 * d.b * 32;
         LACT_LAUNCH("k_update_renorm", "k_update_renorm", 0.0, (k_update_renorm<T>), rowgrid, dim3(256), s, p);
       }
       ++ver;
@@ -721,6 +771,7 @@ struct Runner {
     float* gw_side[2] = {scr<float>(P.t_gwside[0]), scr<float>(P.t_gwside[1])};
     bool side_valid[2] = {false, false};
     hipEvent_t free_ev[2] = {nullptr, nullptr};
+    hipEvent_t dw_done[2] = {nullptr, nullptr};   // newest weight-gradient kernel of the apply steps per buffer
     bool side_used = false;
     float* partial_side = scr<float>(P.t_partial_side);
     int ver = P.nupd, u = P.nupd;
@@ -743,14 +794,6 @@ struct Runner {
         HiddenParams hp = hidden_params(T_, qc, d.q_ld, d.q_bs, gc, d.do_ld, d.do_bs, ver);
         hp.O0 = h(0); hp.O1 = h(1); hp.O2 = h(2);
         launch_hidden(2, hp, ver, T_);
-        {  // dq = gY0 W0 + gY2 W2
-          auto p = row_params<2>();
-          set_term(p.t[0], h(1), d.dh, hbs(), wc(ver, 0), d.d, P.g.elems, d.dh);
-          set_term(p.t[1], h(2), d.dh, hbs(), wc(ver, 2), d.d, P.g.elems, d.dh);
-          p.M = T_; p.N = d.d; p.out = dq + (size_t)st.start * d.d; p.ldo = d.d; p.bso = (long long)d.q_len * d.d;
-          p.accumulate = seen_q.accumulate(st.start, st.end);
-          launch_row_gemm<T, false, 2, EPI_STORE>("apply_bwd_dq", p, d.b, s, true);
-        }
         TokenReduceJob jobs[3];
         memset(jobs, 0, sizeof(jobs));
         jobs[0].nterms = jobs[1].nterms = jobs[2].nterms = 1;
@@ -763,6 +806,16 @@ struct Runner {
         if (!token_reduce("apply_bwd_dw", jobs, T_, sp, gw_side[sb], gw_side[sb], side_valid[sb] ? 1.f : 0.f))
           LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, gw_side[sb], side_valid[sb] ? gw_side[sb] : nullptr, 1.f, partial_side, sp.n, (long long)P.mat3);
         side_valid[sb] = true;
+        dw_done[sb] = side ? side->event() : nullptr;
+        if (dw_done[sb] && s_side != s_main) (void)hipEventRecord(dw_done[sb], s_side);
+        {  // dq = gY0 W0 + gY2 W2
+          auto p = row_params<2>();
+          set_term(p.t[0], h(1), d.dh, hbs(), wc(ver, 0), d.d, P.g.elems, d.dh);
+          set_term(p.t[1], h(2), d.dh, hbs(), wc(ver, 2), d.d, P.g.elems, d.dh);
+          p.M = T_; p.N = d.d; p.out = dq + (size_t)st.start * d.d; p.ldo = d.d; p.bso = (long long)d.q_len * d.d;
+          p.accumulate = seen_q.accumulate(st.start, st.end);
+          launch_row_gemm<T, false, 2, EPI_STORE>("apply_bwd_dq", p, d.b, s, true);
+        }
         continue;
       }
       // ---- update u-1: weights ver-1 -> ver
@@ -776,7 +829,8 @@ struct Runner {
         p.gy = gw_valid ? gwcur : nullptr;
         const int sb = ver & 1;
         if (side_valid[sb]) {
-          wait_for(s_main, s_side);
+          // wait for the apply steps' weight gradients only (their dq GEMMs may still be running)
+          if (dw_done[sb] && s_side != s_main) (void)hipStreamWaitEvent(s_main, dw_done[sb], 0);
           p.gy2 = gw_side[sb];
         }
         p.carry_in = (d.prenorm && carry_main >= 0) ? scr<float>(P.t_gwhat[carry_main]) : nullptr;
@@ -798,6 +852,19 @@ struct Runner {
         const long long xe = (long long)r * c, se = (long long)r * r;
         TN* sg = scr<TN>(P.t_sg);
         TN* gas = scr<TN>(P.t_gas);
+        if (ns_fused_ok()) {
+          if constexpr (kNsBf16) {
+            NsFusedParams f;
+            memset(&f, 0, sizeof(f));
+            f.xb = xb(u, 0); f.xb_it_stride = (long long)P.mat3;
+            f.ab = ab(u, 0); f.bb = bb(u, 0); f.sq_it_stride = (long long)sq3();
+            f.gxf[0] = scr<float>(P.t_gxf[0]); f.gxf[1] = scr<float>(P.t_gxf[1]);
+            f.gxb[0] = scr<uint16_t>(P.t_gxb[0]); f.gxb[1] = scr<uint16_t>(P.t_gxb[1]);
+            f.sg = reinterpret_cast<uint16_t*>(sg); f.gas = reinterpret_cast<uint16_t*>(gas);
+            launch_ns_fused<true>(f);
+            cur = P.S & 1;
+          }
+        } else
         for (int it = P.S - 1; it >= 0; --it) {
           const float ca = P.coeffs[3 * it], cb = P.coeffs[3 * it + 1], cc = P.coeffs[3 * it + 2];
           TN* gb = scr<TN>(P.t_gxb[cur]);
@@ -845,6 +912,7 @@ struct Runner {
         p.mbar = P.momentum ? mbar(u) : nullptr;
         p.gc = scr<T>(P.t_gc);
         p.mdot_part = scr<float>(P.t_mdot);
+        if (P.muon && ns_fused_ok()) p.poison = scr<unsigned>(P.t_nssync) + (size_t)3 * d.b * 32;
         LACT_LAUNCH("k_grad_prep", "k_grad_prep", 0.0, (k_grad_prep<T, TN>), dim3(P.nblk, 3 * d.b), dim3(256), s, p);
         if (P.momentum) {
           gm_valid = true;
@@ -997,10 +1065,12 @@ extern "C" {
 const char* lact_last_error(void) { return g_err.c_str(); }
 int lact_version(void) { return 1; }
 
-int lact_set_stream_overlap(int on) {
+int lact_set_option(int32_t option, int32_t value) {
   std::lock_guard<std::mutex> lock(g_enqueue_mutex);
-  const int was = g_overlap ? 1 : 0;
-  g_overlap = on != 0;
+  bool* flag = option == LACT_OPT_STREAM_OVERLAP ? &g_overlap : (option == LACT_OPT_FUSED_NEWTON_SCHULZ ? &g_fused_ns : nullptr);
+  if (!flag) return fail("lact_set_option: unknown option");
+  const int was = *flag ? 1 : 0;
+  *flag = value != 0;
   return was;
 }
 

@@ -1,0 +1,210 @@
+// Newton-Schulz iterations (forward, and their backward) as ONE launch per batch of matrices.
+//
+// The unfused path runs three dependent GEMM kernels per iteration over 48 small matrices: 6 K-steps of
+// matrix work per block between a launch gap and a cache write-back, 30 launches per update step.  Here the
+// blocks that own the tiles of one matrix stay resident, run the stages back to back and meet at a barrier
+// of their own between stages:
+//
+//   * the block -> tile map gives all tiles of a matrix linear ids that are congruent mod 8, i.e. the same
+//     XCD (workgroups are dealt to the 8 XCDs round-robin), so everything the group exchanges lives in one L2;
+//   * a stage's stores are complete in that L2 once the block has waited for them (vmcnt) -- no L2
+//     write-back is needed inside an XCD -- and the operands written by the partner blocks are read with
+//     device-scope loads that miss the (non-coherent) vector L1;
+//   * the barrier is a counter in that L2: arrive = atomic add, wait = poll (measured ~1.3 us per barrier
+//     against ~4.5 us of launch gap plus the write-back of everything the kernel stored).
+//
+// Should the hardware place a group's blocks on different XCDs (each block publishes its XCC id at the
+// start and the group checks), the group falls back to device-scope release/acquire fences around every
+// barrier -- correct anywhere, only slower.  Every poll loop is bounded: on a timeout the block raises
+// the error word and moves on, so that all waves always exit.
+//
+// Deadlock freedom needs each group to become resident as a whole.  The host launches at most 256 blocks
+// (one per compute unit at this LDS size) per kernel and orders fused launches of one process after each
+// other with an event, so two such kernels never hold compute units while waiting for each other.
+#pragma once
+#include "gemm_dma_kernels.h"
+
+// Optional in-kernel timestamps (defined only by timing experiments; expands to nothing in the library).
+#ifndef LACT_NS_TS
+#define LACT_NS_TS(i)
+#endif
+
+namespace lact {
+
+constexpr int NS_FUSED_MAX_STEPS = 8;
+constexpr long long NS_FUSED_SPIN_LIMIT = 4000000;   // polls of ~64 clocks: a fraction of a second
+
+struct NsFusedParams {
+  int n, z0;                 // matrices of this launch: global indices z0 .. z0+n-1 of the packed [3b] arrays
+  int r, c, S;               // Newton-Schulz orientation [r, c], r <= c, both multiples of 192; iterations
+  int nb, mask, plain;       // u_out is written transposed for matrices whose (z / nb) bit of mask is set
+  float coeffs[3 * NS_FUSED_MAX_STEPS];
+  // forward:  X_0 in xf[0] (fp32) and xb (bf16);  saves X_k, A_k, B_k (bf16) per iteration
+  float* xf[2];
+  uint16_t* xb; long long xb_it_stride;            // X_k at xb + k * xb_it_stride, k < S
+  uint16_t* ab; uint16_t* bb; long long sq_it_stride;
+  uint16_t* xb_last;                               // bf16 copy of X_S (scratch)
+  float* u_out;                                    // X_S, fp32, original orientation
+  // backward: incoming gradient in gxf[0] / gxb[0]; the result ends in gxf[S & 1]
+  float* gxf[2]; uint16_t* gxb[2]; uint16_t* sg; uint16_t* gas;
+  unsigned* sync;            // [n][32] words, zeroed before the launch: word 0 = arrivals, word 1 = XCC id mask
+  unsigned* error;           // set to 1 by a block whose barrier timed out
+};
+
+struct GroupBarrier {
+  unsigned* ctr;
+  unsigned members, epoch;
+  bool split;                // group spread over several XCDs: fence at device scope
+  __device__ __forceinline__ void init(unsigned* line, unsigned nmembers, unsigned* error) {
+    ctr = line; members = nmembers; epoch = 0; split = false;
+    unsigned xcc = 0;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    if (threadIdx.x == 0) __hip_atomic_fetch_or(line + 1, 1u << (xcc & 0xf), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    sync(error, true);
+    unsigned m = __hip_atomic_load(line + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    split = (m & (m - 1)) != 0;
+  }
+  // all threads of the block call it
+  __device__ __forceinline__ void sync(unsigned* error, bool heavy = false) {
+    __syncthreads();   // every wave has waited for its stores before it gets here
+    if (threadIdx.x == 0) {
+      const bool fence = heavy || split;
+      if (fence) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+      __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const unsigned target = members * (++epoch);
+      long long spins = 0;
+      while (__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+        __builtin_amdgcn_s_sleep(1);
+        if (++spins > NS_FUSED_SPIN_LIMIT) {
+          __hip_atomic_store(error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+      }
+      if (fence) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    } else {
+      ++epoch;
+    }
+    __syncthreads();
+  }
+};
+
+template <int NT>
+__device__ __forceinline__ RowGemmDmaParams<NT> ns_row_params() {
+  RowGemmDmaParams<NT> q;
+  q.g.accumulate = 0; q.g.aux = nullptr; q.g.ldaux = 0; q.g.bsaux = 0; q.g.alpha = 1.f; q.g.beta = 0.f;
+  q.g.out_c = nullptr; q.g.out_t = nullptr; q.g.transpose_mask = 0; q.g.nb = 1; q.g.round_out_bf16 = 0;
+  q.out_ct = nullptr;
+  return q;
+}
+__device__ __forceinline__ void ns_term(RowGemmTerm& t, const void* A, int lda, long long bsA, const void* B, int ldb, long long bsB, int K) {
+  t.A = A; t.lda = lda; t.bsA = bsA; t.B = B; t.ldb = ldb; t.bsB = bsB; t.K = K;
+}
+
+// BWD = false: S iterations  A = X X^T;  B = b A + c A A;  X' = a X + B X
+// BWD = true:  the same iterations backwards:  Sg = G X^T + X G^T;  H = b Sg + c (Sg A + A Sg);  G' = a G + B G + H X
+template <bool BWD>
+__global__ __launch_bounds__(DMA_THREADS) void k_ns_fused(const NsFusedParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  using TS = TS_NS;
+  const int tr = p.r / TS::BM, tc = p.c / TS::BN;
+  const int nbm = tr * tc;                           // blocks per matrix
+  const int L = blockIdx.x, j = L >> 3;
+  const int group = (L & 7) + 8 * (j / nbm), member = j % nbm;
+  if (group >= p.n) return;
+  const int z = p.z0 + group;
+  GroupBarrier bar;
+  bar.init(p.sync + (size_t)group * 32, nbm, p.error);
+  const bool sq_tile = member < tr * tr;             // this block owns a tile of the r x r stages
+  const int sx = member / tr, sy = member % tr;      // its tile there
+  const int rx = member / tc, ry = member % tc;      // its tile of the r x c stages
+
+  LACT_NS_TS(0);
+  for (int step = 0; step < p.S; ++step) {
+    const int it = BWD ? p.S - 1 - step : step;
+    // r and c are made opaque once per iteration: otherwise the compiler hoists every stage's loop-invariant
+    // per-lane address registers out of this loop, keeps them all live and spills
+    int r = p.r, c = p.c;
+    asm volatile("" : "+s"(r), "+s"(c));
+    const long long xe = (long long)r * c, se = (long long)r * r;
+    const float ca = p.coeffs[3 * it], cb = p.coeffs[3 * it + 1], cc = p.coeffs[3 * it + 2];
+    const uint16_t* X = p.xb + it * p.xb_it_stride;
+    uint16_t* A = p.ab + it * p.sq_it_stride;
+    uint16_t* B = p.bb + it * p.sq_it_stride;
+    if (!BWD) {
+      const bool last = it + 1 == p.S;
+      if (sq_tile) {
+        auto q = ns_row_params<1>();
+        ns_term(q.g.t[0], X, c, xe, X, c, xe, c);
+        q.g.M = r; q.g.N = r; q.g.out = A; q.g.ldo = r; q.g.bso = se;
+        row_gemm_tile<TS, 1, EPI_STORE, false, true>(q, sx, sy, z, smem);
+      }
+      LACT_NS_TS(1 + step * 6 + 0);
+      bar.sync(p.error);
+      LACT_NS_TS(1 + step * 6 + 1);
+      if (sq_tile) {
+        auto q = ns_row_params<1>();
+        ns_term(q.g.t[0], A, r, se, A, r, se, r);
+        q.g.M = r; q.g.N = r; q.g.out = B; q.g.ldo = r; q.g.bso = se;
+        q.g.aux = A; q.g.ldaux = r; q.g.bsaux = se; q.g.alpha = cc; q.g.beta = cb;
+        row_gemm_tile<TS, 1, EPI_AXPBY, false, true>(q, sx, sy, z, smem);
+      }
+      LACT_NS_TS(1 + step * 6 + 2);
+      bar.sync(p.error);
+      LACT_NS_TS(1 + step * 6 + 3);
+      {
+        auto q = ns_row_params<1>();
+        ns_term(q.g.t[0], B, r, se, X, c, xe, r);
+        q.g.M = r; q.g.N = c; q.g.ldo = c; q.g.bso = xe;
+        q.g.aux = p.xf[it & 1]; q.g.ldaux = c; q.g.bsaux = xe; q.g.alpha = 1.f; q.g.beta = ca;
+        q.g.round_out_bf16 = p.plain;
+        q.g.out = last ? nullptr : p.xf[(it + 1) & 1];
+        q.g.out_c = last ? p.xb_last : p.xb + (it + 1) * p.xb_it_stride;
+        q.g.out_t = last ? p.u_out : nullptr;
+        q.g.transpose_mask = p.mask; q.g.nb = p.nb;
+        row_gemm_tile<TS, 1, EPI_AXPBY_F32_DUAL, true, true>(q, rx, ry, z, smem);
+      }
+      LACT_NS_TS(1 + step * 6 + 4);
+      bar.sync(p.error);
+      LACT_NS_TS(1 + step * 6 + 5);
+    } else {
+      const int cur = step & 1;
+      const uint16_t* gb = p.gxb[cur];
+      if (sq_tile) {   // Sg = G X^T + X G^T
+        auto q = ns_row_params<2>();
+        ns_term(q.g.t[0], gb, c, xe, X, c, xe, c);
+        ns_term(q.g.t[1], X, c, xe, gb, c, xe, c);
+        q.g.M = r; q.g.N = r; q.g.out = p.sg; q.g.ldo = r; q.g.bso = se;
+        row_gemm_tile<TS, 2, EPI_STORE, false, true>(q, sx, sy, z, smem);
+      }
+      LACT_NS_TS(1 + step * 6 + 0);
+      bar.sync(p.error);
+      LACT_NS_TS(1 + step * 6 + 1);
+      if (sq_tile) {   // H = b Sg + c (Sg A + A Sg)
+        auto q = ns_row_params<2>();
+        ns_term(q.g.t[0], p.sg, r, se, A, r, se, r);
+        ns_term(q.g.t[1], A, r, se, p.sg, r, se, r);
+        q.g.M = r; q.g.N = r; q.g.out = p.gas; q.g.ldo = r; q.g.bso = se;
+        q.g.aux = p.sg; q.g.ldaux = r; q.g.bsaux = se; q.g.alpha = cc; q.g.beta = cb;
+        row_gemm_tile<TS, 2, EPI_AXPBY, false, true>(q, sx, sy, z, smem);
+      }
+      LACT_NS_TS(1 + step * 6 + 2);
+      bar.sync(p.error);
+      LACT_NS_TS(1 + step * 6 + 3);
+      {                // G' = a G + B G + H X
+        auto q = ns_row_params<2>();
+        ns_term(q.g.t[0], B, r, se, gb, c, xe, r);
+        ns_term(q.g.t[1], p.gas, r, se, X, c, xe, r);
+        q.g.M = r; q.g.N = c; q.g.ldo = c; q.g.bso = xe;
+        q.g.aux = p.gxf[cur]; q.g.ldaux = c; q.g.bsaux = xe; q.g.alpha = 1.f; q.g.beta = ca;
+        q.g.out = p.gxf[cur ^ 1];
+        q.g.out_c = p.gxb[cur ^ 1];
+        row_gemm_tile<TS, 2, EPI_AXPBY_F32_DUAL, true, true>(q, rx, ry, z, smem);
+      }
+      LACT_NS_TS(1 + step * 6 + 4);
+      bar.sync(p.error);
+      LACT_NS_TS(1 + step * 6 + 5);
+    }
+  }
+}
+
+}  // namespace lact

@@ -192,6 +192,7 @@ struct RenormParams {
   float* main_out;                 // un-normalised accumulator (pre-norm) or null
   float* wf_out; void* wc_out;     // new weights: fp32 state and compute-type copy (may be null)
   float* w_ext[3];                 // caller's weight outputs [b][elems] (same values as wf_out), each nullable
+  const unsigned* poison;          // nonzero word: an earlier kernel of this step failed (barrier timeout) -> results become NaN
   // backward only
   const float* gy;                 // gradient w.r.t. the new weights, or null (= zero)
   const float* gy2;                // second addend of the same gradient (the apply steps' share), or null
@@ -245,12 +246,14 @@ __global__ void k_update_renorm(const RenormParams p) {
     ss += dot4(v, v);
   }
   ss = wave_sum(ss);
-  const float den = sqrtf(ss) + 1e-5f;
+  float den = sqrtf(ss) + 1e-5f;
+  if (p.poison && *p.poison) den = __uint_as_float(0x7fc00000u);
   const float n0 = p.weight_norm ? p.n0[(size_t)z * p.g.maxrows() + row] : 1.f;
   auto emit = [&](int c, const float4& v) {
     if (p.main_out) st4(p.main_out + o + c, v);
     // same operation order as the reference: (w / (norm + eps)) * w_norm
-    const float4 y = p.weight_norm ? f4((v.x / den) * n0, (v.y / den) * n0, (v.z / den) * n0, (v.w / den) * n0) : v;
+    const float4 y = p.weight_norm ? f4((v.x / den) * n0, (v.y / den) * n0, (v.z / den) * n0, (v.w / den) * n0)
+                                   : f4(v.x + 0.f * den, v.y + 0.f * den, v.z + 0.f * den, v.w + 0.f * den);
     st4(p.wf_out + o + c, y);
     if (ext) st4(ext + c, y);
     if (p.wc_out) Elem<T>::store4(reinterpret_cast<T*>(p.wc_out) + o + c, y.x, y.y, y.z, y.w);
@@ -348,6 +351,7 @@ struct GradPrepParams {
   const float* m_prev; const float* mbar;   // null without momentum
   void* gc;                          // [3b][elems] compute-type copy of d loss / d dw  (GEMM operand)
   float* mdot_part;                  // [3b][gridDim.x] partial <g, m_prev>
+  const unsigned* poison;            // nonzero word: an earlier kernel of this step failed (barrier timeout) -> results become NaN
 };
 template <typename T, typename TN>
 __global__ void k_grad_prep(const GradPrepParams p) {
@@ -360,6 +364,7 @@ __global__ void k_grad_prep(const GradPrepParams p) {
     const float n = p.norms[z];
     c0 = 1.f / (n + 1e-7f);
     c1 = n > 0.f ? dot / (n * (n + 1e-7f) * (n + 1e-7f)) : 0.f;
+    if (p.poison && *p.poison) c0 = __uint_as_float(0x7fc00000u);
   }
   const float mb = p.mbar ? p.mbar[ib] : 0.f;
   const FlatRange R(p.g.elems);

@@ -462,15 +462,48 @@ def test_stream_overlap_is_bit_identical(prenorm):
         torch.cuda.synchronize()
         return res
     L_ = _lib.lib()
-    prev = L_.lact_set_stream_overlap(1)
+    prev = L_.lact_set_option(_lib.OPT_STREAM_OVERLAP, 1)
     try:
         on = run()
-        L_.lact_set_stream_overlap(0)
+        L_.lact_set_option(_lib.OPT_STREAM_OVERLAP, 0)
         off = run()
     finally:
-        L_.lact_set_stream_overlap(prev)
+        L_.lact_set_option(_lib.OPT_STREAM_OVERLAP, prev)
     for (o1, g1), (o0, g0) in zip(on, off):
         assert torch.equal(o1, o0)
         for n in g0:
             assert torch.equal(g1[n], g0[n]), n
     assert torch.equal(on[0][0], on[2][0]) and all(torch.equal(on[0][1][n], on[2][1][n]) for n in on[0][1])
+
+
+def test_fused_newton_schulz_is_bit_identical():
+    """All Newton-Schulz iterations of an update as one kernel with per-matrix barriers (rows, columns multiples
+    of 192) against three GEMM launches per iteration: same tile code, same order, so the same bits -- forward
+    and backward, with the apply steps running beside them on the second stream."""
+    say("fused Newton-Schulz on/off")
+    from lact_amd import _lib
+    b, L, d, dh, C = 5, 3 * 256, 384, 192, 256          # w1 is held transposed ([192, 384]); 15 matrices: a partial group of 8
+    inp = problem(b, L, d, dh, seed=91, act=torch.bfloat16)
+    go = torch.randn(b, L, d, generator=torch.Generator().manual_seed(6)).bfloat16().to(DEV)
+
+    def run():
+        res = []
+        for _ in range(2):
+            t = clone_to(inp, DEV)
+            out = T.block_causal_lact_swiglu(*args9(t), C, True, t["momentum"])
+            res.append((out, grads_of(out, t, go)))
+        torch.cuda.synchronize()
+        return res
+    L_ = _lib.lib()
+    prev = L_.lact_set_option(_lib.OPT_FUSED_NEWTON_SCHULZ, 1)
+    try:
+        on = run()
+        L_.lact_set_option(_lib.OPT_FUSED_NEWTON_SCHULZ, 0)
+        off = run()
+    finally:
+        L_.lact_set_option(_lib.OPT_FUSED_NEWTON_SCHULZ, prev)
+    for (o1, g1), (o0, g0) in zip(on, off):
+        assert torch.isfinite(o1.float()).all()
+        assert torch.equal(o1, o0)
+        for n in g0:
+            assert torch.equal(g1[n], g0[n]), n
