@@ -32,9 +32,6 @@ __device__ __forceinline__ uint32_t lds_addr(const void* p) {
 // by another compute unit during this same kernel (the L1 is not coherent with other units' stores).
 template <bool SC1 = false>
 __device__ __forceinline__ void dma16(const void* sbase, uint32_t voff, uint32_t lds_base) {
-#ifdef LACT_EXP_NO_DMA
-  return;
-#endif
   if (SC1)
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 sc1\n\t" ::"s"(lds_base), "v"(voff), "s"(sbase)
                  : "memory", "m0");
@@ -315,9 +312,7 @@ struct DmaPipe {
     // so that the reads spread under the matrix work instead of piling up in front of a wait.
     constexpr int READS = (A_KS ? 2 : 1) * TS::TM + (B_KS ? 2 : 1) * NB * TS::TN, MFMAS = NB * TS::TM * TS::TN;
     auto interleave = [&]() {
-#ifndef LACT_EXP_NO_SCHED
       sched_interleave<READS, MFMAS>();
-#endif
     };
     __syncthreads();
     st = smem + (step % STAGES) * SM::STAGE;

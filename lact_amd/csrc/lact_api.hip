@@ -149,12 +149,20 @@ int ceil_div(int a, int b) { return (a + b - 1) / b; }
 struct Split {
   int n, len;
 };
-Split choose_split(int tokens, int tiles_total) {
+// max_n: slots the partial-sum buffer holds for this launch
+Split choose_split(int tokens, int tiles_total, int max_n) {
   // one split once the tiles alone occupy most of the 256 compute units: the partial sums then never exist
   int ns = tiles_total >= 160 ? 1 : std::max(1, ceil_div(512, std::max(1, tiles_total)));
-  ns = std::min(ns, std::max(1, tokens / 128));
+  ns = std::min(std::min(ns, std::max(1, max_n)), std::max(1, tokens / 128));
   int len = ceil_div(ceil_div(tokens, ns), 64) * 64;
   return Split{ceil_div(tokens, len), len};
+}
+
+// output tiles per matrix of the asynchronous-copy token reduction
+int token_reduce_dma_tiles(int d, int dh) {
+  const bool big = d % TS_NS::BM == 0 && dh % TS_NS::BM == 0;
+  return big ? (d / TS_NS::BM) * (dh / TS_NS::BN)
+             : std::max(ceil_div(dh, TS_SQ::BM) * ceil_div(d, TS_SQ::BN), ceil_div(d, TS_SQ::BM) * ceil_div(dh, TS_SQ::BN));
 }
 
 struct Plan {
@@ -220,7 +228,9 @@ struct Plan {
     lr_slots = ceil_div(d.dh, 128) * 4;   // (hidden tiles) x (wave columns) of the widest update-backward tiling
     tiles = ceil_div(d.dh, TSA::BM) * ceil_div(d.d, TSA::BN);
     tiles = std::max(tiles, ceil_div(d.d, TSA::BM) * ceil_div(d.dh, TSA::BN));
-    nsplit_max = choose_split(Tcap, tiles * 3 * d.b).n;
+    // partial-sum slots: the larger split count of the two token-reduction kernels at the longest chunk (the
+    // count grows with the tokens) + the slot of a ragged tail
+    nsplit_max = std::max(choose_split(Tcap, tiles * 3 * d.b, 16).n, choose_split(Tcap, token_reduce_dma_tiles(d.d, d.dh) * 3 * d.b, 16).n) + 1;
 
     Bump sv;
     s_n0 = sv.take((size_t)3 * d.b * g.maxrows() * 4);
@@ -496,27 +506,35 @@ struct Runner {
     return p;
   }
 
-  // Returns true when the result went straight to `add_out` (= coeff*add_in + sum; single split on the
-  // asynchronous-copy kernel); otherwise the partials are in the scratch slots and the caller reduces them.
-  bool token_reduce(const char* site, const TokenReduceJob (&jobs)[3], int tokens, Split sp, float* add_out = nullptr,
-                    const float* add_in = nullptr, float coeff = 0.f) const {
+  // The three token-reduction GEMMs of a step.  Returns the number of partial-sum slots written to the scratch
+  // buffer (the caller reduces them), or 0 when the result went straight to `add_out` = coeff*add_in + sum.
+  // bf16: whole blocks of 64 tokens run on the asynchronous-copy kernel (straight to add_out when one split
+  // covers them); a ragged tail of fewer than 64 tokens goes through the generic kernel and is added.
+  int token_reduce(const char* site, const TokenReduceJob (&jobs)[3], int tokens, float* add_out = nullptr,
+                   const float* add_in = nullptr, float coeff = 0.f) const {
     TokenReduceParams p;
     memset(&p, 0, sizeof(p));
     for (int i = 0; i < 3; ++i) p.job[i] = jobs[i];
-    p.nb = d.b; p.tokens = tokens; p.split_len = sp.len;
-    p.partial = scr<float>(partial_sel); p.mat_elems = P.g.elems;
+    p.nb = d.b; p.mat_elems = P.g.elems;
+    float* partial = scr<float>(partial_sel);
+    const dim3 flat((unsigned)((P.mat3 / 4 + 255) / 256));
+    int main_tokens = 0, slots = 0;
+    bool direct = false;
     if constexpr (kBf16) {
-      if (sp.len % 64 == 0 && tokens % 64 == 0 && d.d % 8 == 0 && d.dh % 8 == 0) {
+      if (tokens >= 64 && d.d % 8 == 0 && d.dh % 8 == 0) main_tokens = tokens / 64 * 64;
+      if (main_tokens > 0) {
         const bool big = d.d % TS_NS::BM == 0 && d.dh % TS_NS::BM == 0;
-        const int tiles = big ? (d.d / TS_NS::BM) * (d.dh / TS_NS::BN)
-                              : std::max(ceil_div(d.dh, TS_SQ::BM) * ceil_div(d.d, TS_SQ::BN), ceil_div(d.d, TS_SQ::BM) * ceil_div(d.dh, TS_SQ::BN));
+        const int tiles = token_reduce_dma_tiles(d.d, d.dh);
+        const Split sp = choose_split(main_tokens, tiles * 3 * d.b, P.nsplit_max - 1);
         TokenReduceDmaParams pd;
         static_cast<TokenReduceParams&>(pd) = p;
+        pd.tokens = main_tokens; pd.split_len = sp.len; pd.partial = partial;
         pd.map = make_tile_map(sp.n, tiles, 3 * d.b);
         dim3 g(pd.map.grid());
-        const double fl = 6.0 * tokens * d.d * d.dh * d.b * jobs[0].nterms;
-        const bool direct = add_out && sp.n == 1;
+        const double fl = 6.0 * main_tokens * d.d * d.dh * d.b * jobs[0].nterms;
+        direct = add_out && sp.n == 1;
         if (direct) { pd.add_out = add_out; pd.add_in = coeff != 0.f ? add_in : nullptr; pd.coeff = coeff; }
+        else slots = sp.n;
         if (big) {
           constexpr int SM = cmax(DmaSmem<TS_NS, 1, row_stages<TS_NS>()>::BYTES, StageTile<TS_NS, 4>::BYTES);
           static bool once = (allow_big_lds(k_token_reduce_dma<TS_NS>, SM), true);
@@ -528,12 +546,27 @@ struct Runner {
           (void)once;
           LACT_LAUNCH_SMEM("k_token_reduce_dma<128x128>", site, fl, (k_token_reduce_dma<TS_SQ>), g, dim3(DMA_THREADS), SM, s, pd);
         }
-        return direct;
+        if (main_tokens == tokens) return slots;
       }
     }
+    // generic kernel: everything (fp32, or fewer than 64 tokens) or the ragged tail
+    const int rest = tokens - main_tokens;
+    for (int i = 0; i < 3; ++i)
+      for (int t = 0; t < p.job[i].nterms; ++t) {
+        TokenReduceTerm& tt = p.job[i].t[t];
+        tt.A = static_cast<const T*>(tt.A) + (size_t)main_tokens * tt.lda;
+        tt.B = static_cast<const T*>(tt.B) + (size_t)main_tokens * tt.ldb;
+      }
+    const Split sp = main_tokens > 0 ? Split{1, ceil_div(rest, 32) * 32} : choose_split(rest, P.tiles * 3 * d.b, P.nsplit_max - 1);
+    p.tokens = rest; p.split_len = sp.len;
+    p.partial = partial + (size_t)slots * P.mat3;
     dim3 grid(P.tiles, sp.n, 3 * d.b);
-    LACT_LAUNCH("k_token_reduce", site, 6.0 * tokens * d.d * d.dh * d.b * jobs[0].nterms, (k_token_reduce<T, TSA>), grid, dim3(TSA::THREADS), s, p);
-    return false;
+    LACT_LAUNCH("k_token_reduce", site, 6.0 * rest * d.d * d.dh * d.b * jobs[0].nterms, (k_token_reduce<T, TSA>), grid, dim3(TSA::THREADS), s, p);
+    if (direct) {   // add the tail to what the main part wrote
+      LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, add_out, add_out, 1.f, partial, sp.n, (long long)P.mat3);
+      return 0;
+    }
+    return slots + sp.n;
   }
 
   RenormParams renorm_params(int u, int ver_prev) const {
@@ -591,7 +624,7 @@ struct Runner {
         hp.O0 = h(0); hp.O1 = h(1); hp.O2 = h(2);
         launch_hidden(1, hp, ver, T_);
       }
-      const Split sp = choose_split(T_, P.tiles * 3 * d.b);
+      int dw_slots = 0;
       {
         TokenReduceJob jobs[3];
         memset(jobs, 0, sizeof(jobs));
@@ -602,13 +635,13 @@ struct Runner {
         set_tr_term(jobs[1].t[0], vc, d.v_ld, d.v_bs, h(1), d.dh, hbs());
         jobs[2].M = d.dh; jobs[2].N = d.d;
         set_tr_term(jobs[2].t[0], h(2), d.dh, hbs(), kc, d.k_ld, d.k_bs);
-        token_reduce("update_dw", jobs, T_, sp);
+        dw_slots = token_reduce("update_dw", jobs, T_);
       }
       if (P.momentum) LACT_LAUNCH("k_momentum_mean", "k_momentum_mean", 0.0, k_momentum_mean, dim3(d.b), dim3(256), s, mom, (long long)d.kv_len, st.start, T_, mbar(u));
       {
         MomentumPrepParams p;
         memset(&p, 0, sizeof(p));
-        p.g = P.g; p.partial = scr<float>(P.t_partial); p.nsplit = sp.n;
+        p.g = P.g; p.partial = scr<float>(P.t_partial); p.nsplit = dw_slots;
         p.m_prev = (P.momentum && u > 0) ? dsave(u - 1) : nullptr;
         p.mbar = P.momentum ? mbar(u) : nullptr;
         p.d_out = dsave(u);
@@ -780,7 +813,6 @@ struct Runner {
     for (int si = (int)P.steps.size() - 1; si >= 0; --si) {
       const lact_step_t& st = P.steps[si];
       const int T_ = st.end - st.start;
-      const Split sp = choose_split(T_, P.tiles * 3 * d.b);
       if (st.kind == LACT_APPLY) {
         const int sb = ver & 1;
         if (!side_valid[sb] && free_ev[sb] && s_side != s_main) {
@@ -803,8 +835,8 @@ struct Runner {
         set_tr_term(jobs[1].t[0], gc, d.do_ld, d.do_bs, h(0), d.dh, hbs());
         jobs[2].M = d.dh; jobs[2].N = d.d;
         set_tr_term(jobs[2].t[0], h(2), d.dh, hbs(), qc, d.q_ld, d.q_bs);
-        if (!token_reduce("apply_bwd_dw", jobs, T_, sp, gw_side[sb], gw_side[sb], side_valid[sb] ? 1.f : 0.f))
-          LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, gw_side[sb], side_valid[sb] ? gw_side[sb] : nullptr, 1.f, partial_side, sp.n, (long long)P.mat3);
+        if (const int ns_ = token_reduce("apply_bwd_dw", jobs, T_, gw_side[sb], gw_side[sb], side_valid[sb] ? 1.f : 0.f))
+          LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, gw_side[sb], side_valid[sb] ? gw_side[sb] : nullptr, 1.f, partial_side, ns_, (long long)P.mat3);
         side_valid[sb] = true;
         dw_done[sb] = side ? side->event() : nullptr;
         if (dw_done[sb] && s_side != s_main) (void)hipEventRecord(dw_done[sb], s_side);
@@ -965,8 +997,8 @@ struct Runner {
         jobs[2].M = d.dh; jobs[2].N = d.d;
         set_tr_term(jobs[2].t[0], h(2), d.dh, hbs(), kc, d.k_ld, d.k_bs);
         const float pass = d.prenorm ? 0.f : ((P.muon && d.muon_replaces_weight) ? 0.f : 1.f);
-        if (!token_reduce("update_bwd_dw", jobs, T_, sp, gwcur, gwhat, pass))
-          LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, gwcur, pass != 0.f ? gwhat : nullptr, pass, partial, sp.n, (long long)P.mat3);
+        if (const int ns_ = token_reduce("update_bwd_dw", jobs, T_, gwcur, gwhat, pass))
+          LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, gwcur, pass != 0.f ? gwhat : nullptr, pass, partial, ns_, (long long)P.mat3);
         gw_valid = true;
       }
       LACT_LAUNCH("k_lr_reduce", "k_lr_reduce", 0.0, k_lr_reduce, dim3(ceil_div(T_, 256), d.b, 3), dim3(256), s, scr<float>(P.t_lrpart),
