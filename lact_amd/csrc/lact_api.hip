@@ -396,17 +396,23 @@ struct Runner {
     if (side && g_overlap) s_side = side->stream;
   }
   // ---- fused Newton-Schulz: one launch per batch of at most 256 resident blocks
+  static bool tiles_fit(int r, int c, int edge) { return r % edge == 0 && c % edge == 0 && (r / edge) * (c / edge) <= 32; }
+  // 192 x 192 tiles when the matrices fill at least half the chip with them, else 128 x 128 (more, smaller blocks)
+  bool ns_fused_small_tiles() const {
+    if (!tiles_fit(P.r, P.c, 128)) return false;
+    if (!tiles_fit(P.r, P.c, 192)) return true;
+    return 3 * d.b * (P.r / 192) * (P.c / 192) < 128;
+  }
   bool ns_fused_ok() const {
     if (!g_fused_ns || !side || !kNsBf16 || P.S < 1 || P.S > NS_FUSED_MAX_STEPS) return false;
-    if (P.r % TS_NS::BM || P.c % TS_NS::BN) return false;
-    return (P.r / TS_NS::BM) * (P.c / TS_NS::BN) <= 32;
+    return tiles_fit(P.r, P.c, 192) || tiles_fit(P.r, P.c, 128);
   }
-  template <bool BWD>
-  void launch_ns_fused(NsFusedParams p) {
-    constexpr int SM = cmax(DmaSmem<TS_NS, 1, row_stages<TS_NS>()>::BYTES, StageTile<TS_NS, 4>::BYTES);
-    static bool once = (allow_big_lds(k_ns_fused<BWD>, SM), true);
+  template <class TS, bool BWD>
+  void launch_ns_fused_ts(NsFusedParams p) {
+    constexpr int SM = cmax(DmaSmem<TS, 1, row_stages<TS>()>::BYTES, StageTile<TS, 4>::BYTES);
+    static bool once = (allow_big_lds(k_ns_fused<TS, BWD>, SM), true);
     (void)once;
-    const int total = 3 * d.b, nbm = (P.r / TS_NS::BM) * (P.c / TS_NS::BN);
+    const int total = 3 * d.b, nbm = (P.r / TS::BM) * (P.c / TS::BN);
     const int per = (256 / nbm) / 8 * 8;
     unsigned* sync = scr<unsigned>(P.t_nssync);
     const long long words = (long long)total * 32 + 32;
@@ -415,17 +421,23 @@ struct Runner {
     for (int i = 0; i < 3 * P.S; ++i) p.coeffs[i] = P.coeffs[i];
     p.error = sync + (size_t)total * 32;
     const double terms = BWD ? 6.0 : 3.0;
+    static const std::string name = std::string("k_ns_fused<") + std::to_string(TS::BM) + "x" + std::to_string(TS::BN) + (BWD ? ",bwd>" : ",fwd>");
     for (int z0 = 0; z0 < total; z0 += per) {
       p.z0 = z0; p.n = std::min(per, total - z0); p.sync = sync + (size_t)z0 * 32;
       const int grid = 8 * ((p.n + 7) / 8) * nbm;
       // fused launches of this process never overlap each other (each needs its groups resident as a whole)
       if (side->fused_recorded) (void)hipStreamWaitEvent(s, side->fused_done, 0);
-      LACT_LAUNCH_SMEM(BWD ? "k_ns_fused<bwd>" : "k_ns_fused<fwd>", BWD ? "ns_bwd" : "ns_fwd", terms * 2.0 * P.r * P.r * P.c * P.S * p.n,
-                       (k_ns_fused<BWD>), dim3(grid), dim3(DMA_THREADS), SM, s, p);
+      LACT_LAUNCH_SMEM(name.c_str(), BWD ? "ns_bwd" : "ns_fwd", terms * 2.0 * P.r * P.r * P.c * P.S * p.n,
+                       (k_ns_fused<TS, BWD>), dim3(grid), dim3(DMA_THREADS), SM, s, p);
       if (!side->fused_done) (void)hipEventCreateWithFlags(&side->fused_done, hipEventDisableTiming);
       (void)hipEventRecord(side->fused_done, s);
       side->fused_recorded = true;
     }
+  }
+  template <bool BWD>
+  void launch_ns_fused(const NsFusedParams& p) {
+    if (ns_fused_small_tiles()) launch_ns_fused_ts<TS_SQ, BWD>(p);
+    else launch_ns_fused_ts<TS_NS, BWD>(p);
   }
   // `waiter` waits for everything enqueued so far on `on`
   void wait_for(hipStream_t waiter, hipStream_t on) {

@@ -36,7 +36,7 @@ constexpr long long NS_FUSED_SPIN_LIMIT = 4000000;   // polls of ~64 clocks: a f
 
 struct NsFusedParams {
   int n, z0;                 // matrices of this launch: global indices z0 .. z0+n-1 of the packed [3b] arrays
-  int r, c, S;               // Newton-Schulz orientation [r, c], r <= c, both multiples of 192; iterations
+  int r, c, S;               // Newton-Schulz orientation [r, c], r <= c, both multiples of the tile edge; iterations
   int nb, mask, plain;       // u_out is written transposed for matrices whose (z / nb) bit of mask is set
   float coeffs[3 * NS_FUSED_MAX_STEPS];
   // forward:  X_0 in xf[0] (fp32) and xb (bf16);  saves X_k, A_k, B_k (bf16) per iteration
@@ -102,10 +102,10 @@ __device__ __forceinline__ void ns_term(RowGemmTerm& t, const void* A, int lda, 
 
 // BWD = false: S iterations  A = X X^T;  B = b A + c A A;  X' = a X + B X
 // BWD = true:  the same iterations backwards:  Sg = G X^T + X G^T;  H = b Sg + c (Sg A + A Sg);  G' = a G + B G + H X
-template <bool BWD>
+// TS: 192 x 192 tiles, or 128 x 128 when there are too few matrices to fill the chip with the large tile.
+template <class TS, bool BWD>
 __global__ __launch_bounds__(DMA_THREADS) void k_ns_fused(const NsFusedParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  using TS = TS_NS;
   const int tr = p.r / TS::BM, tc = p.c / TS::BN;
   const int nbm = tr * tc;                           // blocks per matrix
   const int L = blockIdx.x, j = L >> 3;

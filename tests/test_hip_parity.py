@@ -476,13 +476,16 @@ def test_stream_overlap_is_bit_identical(prenorm):
     assert torch.equal(on[0][0], on[2][0]) and all(torch.equal(on[0][1][n], on[2][1][n]) for n in on[0][1])
 
 
-def test_fused_newton_schulz_is_bit_identical():
+@pytest.mark.parametrize("b,d,dh", [(5, 384, 192), (2, 384, 384), (3, 256, 128)])
+def test_fused_newton_schulz_is_bit_identical(b, d, dh):
     """All Newton-Schulz iterations of an update as one kernel with per-matrix barriers (rows, columns multiples
     of 192) against three GEMM launches per iteration: same tile code, same order, so the same bits -- forward
     and backward, with the apply steps running beside them on the second stream."""
-    say("fused Newton-Schulz on/off")
+    say("fused Newton-Schulz on/off", b, d, dh)
     from lact_amd import _lib
-    b, L, d, dh, C = 5, 3 * 256, 384, 192, 256          # w1 is held transposed ([192, 384]); 15 matrices: a partial group of 8
+    # (5, 384, 192): w1 is held transposed ([192, 384]), 15 matrices = a partial group of 8, 192-tiles;
+    # (2, 384, 384): few matrices -> 128-tiles, 9 blocks per matrix;  (3, 256, 128): only 128-tiles fit
+    L, C = 3 * 256, 256
     inp = problem(b, L, d, dh, seed=91, act=torch.bfloat16)
     go = torch.randn(b, L, d, generator=torch.Generator().manual_seed(6)).bfloat16().to(DEV)
 
