@@ -9,6 +9,7 @@
 #include <string>
 #include <vector>
 #include <mutex>
+#include <memory>
 
 #include <type_traits>
 
@@ -607,24 +608,39 @@ struct Runner {
       LACT_LAUNCH("k_init_state", "k_init_state", 0.0, (k_init_state<T>), rowgrid, dim3(256), s, p);
     }
     int ver = 0, u = 0;
-    int side_has_ver = -1;     // newest weight version the side stream has been made to wait for
     bool side_used = false;
+    // Apply steps only need their weight version, which is final once they are met in program order.  They are
+    // held back and enqueued on the side stream at the point of the following update where the chip is least
+    // busy -- in front of its Newton-Schulz kernels, which leave a quarter of the compute units idle -- or at
+    // the end of the program.
+    std::vector<std::pair<const lact_step_t*, int>> pending;   // (apply step, weight version)
+    auto flush_applies = [&](bool beside_update) {
+      if (pending.empty()) return;
+      // with no update left to run beside, the caller's stream is the shortest way (no event hand-over)
+      std::unique_ptr<OnSide> on_side;
+      if (beside_update) {
+        wait_for(s_side, s_main);
+        side_used = true;
+        on_side.reset(new OnSide(*this));
+      }
+      for (auto& pa : pending) {
+        const lact_step_t& st = *pa.first;
+        const int T_ = st.end - st.start, av = pa.second;
+        HiddenParams hp = hidden_params(T_, q + (size_t)st.start * d.q_ld, d.q_ld, d.q_bs, nullptr, 0, 0, av);
+        hp.O0 = h(0);
+        launch_hidden(0, hp, av, T_);
+        auto p = row_params<1>();
+        set_term(p.t[0], h(0), d.dh, hbs(), wc(av, 1), d.dh, P.g.elems, d.dh);
+        p.M = T_; p.N = d.d; p.out = out + (size_t)st.out_start * d.o_ld; p.ldo = d.o_ld; p.bso = d.o_bs;
+        launch_row_gemm<T, true, 1, EPI_STORE>("apply_out", p, d.b, s, true);
+      }
+      pending.clear();
+    };
     for (const auto& st : P.steps) {
       const int T_ = st.end - st.start;
       if (st.kind == LACT_APPLY) {
-        if (side_has_ver < ver) {
-          wait_for(s_side, s_main);
-          side_has_ver = ver;
-        }
-        side_used = true;
-        OnSide on_side(*this);
-        HiddenParams hp = hidden_params(T_, q + (size_t)st.start * d.q_ld, d.q_ld, d.q_bs, nullptr, 0, 0, ver);
-        hp.O0 = h(0);
-        launch_hidden(0, hp, ver, T_);
-        auto p = row_params<1>();
-        set_term(p.t[0], h(0), d.dh, hbs(), wc(ver, 1), d.dh, P.g.elems, d.dh);
-        p.M = T_; p.N = d.d; p.out = out + (size_t)st.out_start * d.o_ld; p.ldo = d.o_ld; p.bso = d.o_bs;
-        launch_row_gemm<T, true, 1, EPI_STORE>("apply_out", p, d.b, s, true);
+        pending.emplace_back(&st, ver);
+        if (s_side == s_main) flush_applies(false);   // one stream: plain program order
         continue;
       }
       // ---- update
@@ -664,6 +680,7 @@ struct Runner {
           for (int j = 0; j < 3; ++j) p.m_ext[j] = m_out[j];
         LACT_LAUNCH("k_momentum_prep", "k_momentum_prep", 0.0, (k_momentum_prep<TN>), dim3(P.nblk, 3 * d.b), dim3(256), s, p);
       }
+      flush_applies(true);
       if (P.muon) {
         NsScaleParams p;
         memset(&p, 0, sizeof(p));
@@ -710,6 +727,7 @@ struct Runner {
       ++ver;
       ++u;
     }
+    flush_applies(false);
     if (side_used) wait_for(s_main, s_side);
     // final weights and momentum state: written by the last update's kernels; copied only when no update ran
     const dim3 eg((unsigned)((P.g.elems / 4 + 255) / 256), 3 * d.b);
@@ -818,6 +836,11 @@ struct Runner {
     hipEvent_t free_ev[2] = {nullptr, nullptr};
     hipEvent_t dw_done[2] = {nullptr, nullptr};   // newest weight-gradient kernel of the apply steps per buffer
     bool side_used = false;
+    hipEvent_t main_dq_ev = nullptr;   // a dq GEMM on the side stream still reads the main chain's intermediates
+    auto wait_main_dq = [&]() {
+      if (main_dq_ev) (void)hipStreamWaitEvent(s_main, main_dq_ev, 0);
+      main_dq_ev = nullptr;
+    };
     float* partial_side = scr<float>(P.t_partial_side);
     int ver = P.nupd, u = P.nupd;
     int carry_main = -1;       // index of the gwhat buffer holding the accumulator's gradient (pre-norm)
@@ -826,6 +849,50 @@ struct Runner {
       const lact_step_t& st = P.steps[si];
       const int T_ = st.end - st.start;
       if (st.kind == LACT_APPLY) {
+        const T* qc = q + (size_t)st.start * d.q_ld;
+        const T* gc = dout + (size_t)st.out_start * d.do_ld;
+        auto dw_jobs = [&](TokenReduceJob (&jobs)[3]) {
+          memset(jobs, 0, sizeof(jobs));
+          jobs[0].nterms = jobs[1].nterms = jobs[2].nterms = 1;
+          jobs[0].M = d.dh; jobs[0].N = d.d;
+          set_tr_term(jobs[0].t[0], h(1), d.dh, hbs(), qc, d.q_ld, d.q_bs);
+          jobs[1].M = d.d; jobs[1].N = d.dh;
+          set_tr_term(jobs[1].t[0], gc, d.do_ld, d.do_bs, h(0), d.dh, hbs());
+          jobs[2].M = d.dh; jobs[2].N = d.d;
+          set_tr_term(jobs[2].t[0], h(2), d.dh, hbs(), qc, d.q_ld, d.q_bs);
+        };
+        auto dq_gemm = [&]() {   // dq = gY0 W0 + gY2 W2
+          auto p = row_params<2>();
+          set_term(p.t[0], h(1), d.dh, hbs(), wc(ver, 0), d.d, P.g.elems, d.dh);
+          set_term(p.t[1], h(2), d.dh, hbs(), wc(ver, 2), d.d, P.g.elems, d.dh);
+          p.M = T_; p.N = d.d; p.out = dq + (size_t)st.start * d.d; p.ldo = d.d; p.bso = (long long)d.q_len * d.d;
+          p.accumulate = seen_q.accumulate(st.start, st.end);
+          launch_row_gemm<T, false, 2, EPI_STORE>("apply_bwd_dq", p, d.b, s, true);
+        };
+        if (ver == P.nupd) {
+          // Applies of the newest weight version: the update chain cannot start before their weight gradients,
+          // so they stay on the caller's stream (no event hand-over in the critical path); only dq, which nothing
+          // waits for, goes to the side stream and reads this chain's intermediates.
+          wait_main_dq();
+          HiddenParams hp = hidden_params(T_, qc, d.q_ld, d.q_bs, gc, d.do_ld, d.do_bs, ver);
+          hp.O0 = h(0); hp.O1 = h(1); hp.O2 = h(2);
+          launch_hidden(2, hp, ver, T_);
+          wait_for(s_side, s_main);
+          TokenReduceJob jobs[3];
+          dw_jobs(jobs);
+          if (const int ns_ = token_reduce("apply_bwd_dw", jobs, T_, gwcur, gwcur, gw_valid ? 1.f : 0.f))
+            LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, gwcur, gw_valid ? gwcur : nullptr, 1.f, partial, ns_, (long long)P.mat3);
+          gw_valid = true;
+          s = s_side;
+          dq_gemm();
+          s = s_main;
+          if (side && s_side != s_main) {
+            main_dq_ev = side->event();
+            (void)hipEventRecord(main_dq_ev, s_side);
+            side_used = true;
+          }
+          continue;
+        }
         const int sb = ver & 1;
         if (!side_valid[sb] && free_ev[sb] && s_side != s_main) {
           (void)hipStreamWaitEvent(s_side, free_ev[sb], 0);
@@ -833,33 +900,17 @@ struct Runner {
         }
         side_used = true;
         OnSide on_side(*this);
-        const T* qc = q + (size_t)st.start * d.q_ld;
-        const T* gc = dout + (size_t)st.out_start * d.do_ld;
         HiddenParams hp = hidden_params(T_, qc, d.q_ld, d.q_bs, gc, d.do_ld, d.do_bs, ver);
         hp.O0 = h(0); hp.O1 = h(1); hp.O2 = h(2);
         launch_hidden(2, hp, ver, T_);
         TokenReduceJob jobs[3];
-        memset(jobs, 0, sizeof(jobs));
-        jobs[0].nterms = jobs[1].nterms = jobs[2].nterms = 1;
-        jobs[0].M = d.dh; jobs[0].N = d.d;
-        set_tr_term(jobs[0].t[0], h(1), d.dh, hbs(), qc, d.q_ld, d.q_bs);
-        jobs[1].M = d.d; jobs[1].N = d.dh;
-        set_tr_term(jobs[1].t[0], gc, d.do_ld, d.do_bs, h(0), d.dh, hbs());
-        jobs[2].M = d.dh; jobs[2].N = d.d;
-        set_tr_term(jobs[2].t[0], h(2), d.dh, hbs(), qc, d.q_ld, d.q_bs);
+        dw_jobs(jobs);
         if (const int ns_ = token_reduce("apply_bwd_dw", jobs, T_, gw_side[sb], gw_side[sb], side_valid[sb] ? 1.f : 0.f))
           LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, gw_side[sb], side_valid[sb] ? gw_side[sb] : nullptr, 1.f, partial_side, ns_, (long long)P.mat3);
         side_valid[sb] = true;
         dw_done[sb] = side ? side->event() : nullptr;
         if (dw_done[sb] && s_side != s_main) (void)hipEventRecord(dw_done[sb], s_side);
-        {  // dq = gY0 W0 + gY2 W2
-          auto p = row_params<2>();
-          set_term(p.t[0], h(1), d.dh, hbs(), wc(ver, 0), d.d, P.g.elems, d.dh);
-          set_term(p.t[1], h(2), d.dh, hbs(), wc(ver, 2), d.d, P.g.elems, d.dh);
-          p.M = T_; p.N = d.d; p.out = dq + (size_t)st.start * d.d; p.ldo = d.d; p.bso = (long long)d.q_len * d.d;
-          p.accumulate = seen_q.accumulate(st.start, st.end);
-          launch_row_gemm<T, false, 2, EPI_STORE>("apply_bwd_dq", p, d.b, s, true);
-        }
+        dq_gemm();
         continue;
       }
       // ---- update u-1: weights ver-1 -> ver
@@ -977,6 +1028,7 @@ struct Runner {
         hp.lrpart = scr<float>(P.t_lrpart);
         hp.lrpart_stride = (long long)d.b * P.Tcap;
         hp.lrpart_mat_stride = (long long)P.lr_slots * d.b * P.Tcap;
+        wait_main_dq();
         launch_hidden(3, hp, vprev, T_);
       }
       const bool acc_kv = seen_kv.accumulate(st.start, st.end);
