@@ -371,6 +371,12 @@ struct StageTile {
   __device__ static __forceinline__ bool active() { return (int)threadIdx.x < RPP * LPR; }   // RPP*LPR <= 256: loader wave idle
   __device__ static __forceinline__ int row0() { return threadIdx.x / LPR; }
   __device__ static __forceinline__ int col0() { return (threadIdx.x % LPR) * CH; }
+  // 16 bytes of copy-out pass `ps` for the thread whose first row is r0 (src = its address in pass 0); a pass
+  // that would leave the tile reads pass 0 again (the caller discards it)
+  __device__ static __forceinline__ uint4 read16(const char* src, int r0, int ps) {
+    const bool inside = (ps + 1) * RPP <= TS::BM || r0 + ps * RPP < TS::BM;
+    return *reinterpret_cast<const uint4*>(src + (inside ? ps * RPP * LD * E : 0));
+  }
 };
 
 // Plain copy of a staged bf16 tile to `out` (row stride ld elements), rows/cols = valid extent of the tile.
@@ -383,10 +389,15 @@ __device__ __forceinline__ void copy_out_b16(const char* smem, uint16_t* out, in
   const char* src = smem + (r0 * ST::LD + c0) * 2;
   uint16_t* dst = out + (size_t)r0 * ld + c0;
   const size_t step = (size_t)ST::RPP * ld;
+  uint4 ug[8];
 #pragma unroll
   for (int ps = 0; ps < ST::PASSES; ++ps) {
-    if (r0 + ps * ST::RPP < rows && r0 + ps * ST::RPP < TS::BM)
-      *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(src + ps * ST::RPP * ST::LD * 2);
+    if (ps % 8 == 0) {
+#pragma unroll
+      for (int g = 0; g < 8; ++g)
+        if (ps + g < ST::PASSES) ug[g] = ST::read16(src, r0, ps + g);
+    }
+    if (r0 + ps * ST::RPP < rows && r0 + ps * ST::RPP < TS::BM) *reinterpret_cast<uint4*>(dst) = ug[ps % 8];
     dst += step;
   }
 }

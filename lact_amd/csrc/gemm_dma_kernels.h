@@ -89,11 +89,18 @@ __device__ __forceinline__ void row_gemm_tile(const RowGemmDmaParams<NT>& pp, in
         }
       }
       const float al = EPI == EPI_STORE ? 1.f : p.alpha, be = EPI == EPI_STORE ? 1.f : p.beta;
+      // LDS reads in unconditional groups of 8 (a branch per row would put every read's latency in line)
+      uint4 ug[8];
 #pragma unroll
       for (int ps = 0; ps < ST::PASSES; ++ps) {
+        if (ps % 8 == 0) {
+#pragma unroll
+          for (int g = 0; g < 8; ++g)
+            if (ps + g < ST::PASSES) ug[g] = ST::read16(src, r0, ps + g);
+        }
         const int r = r0 + ps * ST::RPP;
         if (r < TS::BM && m0 + r < p.M) {
-          uint4 u = *reinterpret_cast<const uint4*>(src + ps * ST::RPP * ST::LD * 2);
+          uint4 u = ug[ps % 8];
           if (blend) {
             uint32_t uu[4] = {u.x, u.y, u.z, u.w}, ww[4] = {w[ps].x, w[ps].y, w[ps].z, w[ps].w};
 #pragma unroll
@@ -130,12 +137,18 @@ __device__ __forceinline__ void row_gemm_tile(const RowGemmDmaParams<NT>& pp, in
         const int r = r0 + ps * ST::RPP;
         x4[ps] = (r < TS::BM && m0 + r < p.M) ? *reinterpret_cast<const float4*>(aux + ps * astep) : make_float4(0.f, 0.f, 0.f, 0.f);
       }
+        uint4 ag[8];
 #pragma unroll
       for (int ps = 0; ps < ST::PASSES; ++ps) {
+        if (ps % 8 == 0) {
+#pragma unroll
+          for (int g = 0; g < 8; ++g)
+            if (ps + g < ST::PASSES) ag[g] = ST::read16(src, r0, ps + g);
+        }
         const int r = r0 + ps * ST::RPP;
         if (r < TS::BM && m0 + r < p.M) {
           float4* sp = reinterpret_cast<float4*>(src + ps * ST::RPP * ST::LD * 4);
-          const float4 a4 = *sp;
+          const float4 a4 = __builtin_bit_cast(float4, ag[ps % 8]);
           float v[4] = {p.alpha * a4.x + p.beta * x4[ps].x, p.alpha * a4.y + p.beta * x4[ps].y, p.alpha * a4.z + p.beta * x4[ps].z,
                         p.alpha * a4.w + p.beta * x4[ps].w};
           if (p.round_out_bf16) {
@@ -536,11 +549,17 @@ __global__ __launch_bounds__(DMA_THREADS) void k_token_reduce_dma(const TokenRed
         x4[ps] = (r < TS::BM && m0 + r < job.M) ? *reinterpret_cast<const float4*>(ain + ps * rstep) : make_float4(0.f, 0.f, 0.f, 0.f);
       }
     }
+    uint4 vg[8];
 #pragma unroll
     for (int ps = 0; ps < ST::PASSES; ++ps) {
+      if (ps % 8 == 0) {
+#pragma unroll
+        for (int g = 0; g < 8; ++g)
+          if (ps + g < ST::PASSES) vg[g] = ST::read16(src, r0, ps + g);
+      }
       const int r = r0 + ps * ST::RPP;
       if (r < TS::BM && m0 + r < job.M) {
-        float4 v = *reinterpret_cast<const float4*>(src + ps * ST::RPP * ST::LD * 4);
+        float4 v = __builtin_bit_cast(float4, vg[ps % 8]);
         if (blend) {
           v.x += p.coeff * x4[ps].x; v.y += p.coeff * x4[ps].y; v.z += p.coeff * x4[ps].z; v.w += p.coeff * x4[ps].w;
         }
