@@ -128,7 +128,7 @@ struct TileMap {
   __host__ __device__ int group_size() const { return by_batch ? gx * gy : gy; }
   __host__ __device__ int groups() const { return by_batch ? gz : gz * gx; }
   __host__ __device__ int grid() const { return 8 * ((groups() + 7) / 8) * group_size(); }
-  __device__ __forceinline__ bool locate(int L, int& x, int& y, int& z) const {
+  __host__ __device__ bool locate_host(int L, int& x, int& y, int& z) const {   // same arithmetic, callable from host tests
     const int gs = group_size();
     const int j = L >> 3;
     const int g = (L & 7) + 8 * (j / gs), m = j % gs;
@@ -137,6 +137,7 @@ struct TileMap {
     else { z = g / gx; x = g % gx; y = m; }
     return true;
   }
+  __device__ __forceinline__ bool locate(int L, int& x, int& y, int& z) const { return locate_host(L, x, y, z); }
 };
 inline TileMap make_tile_map(int gx, int gy, int gz) {
   TileMap m;
