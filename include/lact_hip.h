@@ -64,6 +64,9 @@ typedef struct lact_desc {
   int32_t ns_mode;               /* LACT_NS_* */
   int64_t q_bs, k_bs, v_bs, o_bs, do_bs;
   int32_t q_ld, k_ld, v_ld, o_ld, do_ld;
+  /* The two places where the fused-kernel driver differs in semantics (ttt_operation_fused_kernel.py): */
+  int32_t muon_stacked;          /* Newton-Schulz on cat(dw0, dw2) [2dh, d] and on dw1 (:168-170, :308-310) */
+  int32_t renorm_eps_in_sqrt;    /* y = w / sqrt(|w|^2 + eps) * n0 (:172-173; l2norm_triton_kernels.py:205-214) */
 } lact_desc_t;
 
 const char* lact_last_error(void);
@@ -74,7 +77,8 @@ int lact_version(void);
 int lact_query_sizes(const lact_desc_t* desc, size_t* saved_bytes, size_t* scratch_bytes);
 
 /* Whole forward of one program.  Replaces block_causal_lact_swiglu / prenorm_block_causal_lact_swiglu
- * (ttt_operation.py:71-214, 219-364), bidirectional_lact_swiglu (bidirectional_lact_layer.py:74-160),
+ * (ttt_operation.py:71-214, 219-364), their fused-kernel twins (ttt_operation_fused_kernel.py:67-338),
+ * bidirectional_lact_swiglu (bidirectional_lact_layer.py:74-160),
  * fast_weight_swish_glu_weight_norm_mini_batch_apply (lact_ttt.py:71-147) and the
  * ar_fast_weight_swish_glu_weight_norm_mini_batch family (ar_lact_swa_repeat.py:23-296).
  * w_out[3] / m_out[3] (each nullable, fp32, shapes of w0,w1,w2) receive the final fast weights and

@@ -8,6 +8,8 @@ The package mirrors the reference's call signatures for this one path:
 All arithmetic runs in lib/liblact_hip.so (built from csrc/ with hipcc for gfx950)."""
 from .ops import NS5_COEFFS, NS_CLASSIC, Program, block_causal_steps, run_program  # noqa: F401
 from .ttt_operation import (block_causal_lact_swiglu, l2_norm, prenorm_block_causal_lact_swiglu,  # noqa: F401
+                            postnorm_block_causal_lact_swiglu_fused_kernel_triton,
+                            prenorm_block_causal_lact_swiglu_fused_kernel_triton,
                             silu_backprop, zeropower_via_newtonschulz5)
 from .minimal import bidirectional_lact_swiglu, inv_softplus  # noqa: F401
 from .nvs import TTTOperator, fast_weight_swish_glu_weight_norm_mini_batch_apply  # noqa: F401

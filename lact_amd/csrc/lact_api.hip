@@ -166,8 +166,18 @@ int token_reduce_dma_tiles(int d, int dh) {
              : std::max(ceil_div(dh, TS_SQ::BM) * ceil_div(d, TS_SQ::BN), ceil_div(d, TS_SQ::BM) * ceil_div(dh, TS_SQ::BN));
 }
 
+// One Newton-Schulz launch group: n matrices of one geometry, laid out one after the other.
+struct NsBatch {
+  int n, r, c;          // matrices, Newton-Schulz orientation [r, c] (r <= c)
+  int mask, nb;         // the orthogonalised update of matrix z is written back transposed when bit (z / nb) of mask is set
+  int first;            // index of its first matrix among all Newton-Schulz matrices (barrier lines)
+  size_t xoff, sqoff;   // element offsets: [r, c]-shaped buffers (and the update in original orientation); [r, r]-shaped buffers
+};
+
 struct Plan {
   lact_desc_t d;
+  std::vector<NsBatch> nsb;
+  size_t sq_total = 0;    // elements of one [r, r]-shaped buffer over all batches
   std::vector<lact_step_t> steps;
   std::vector<float> coeffs;
   MatGeom g;
@@ -225,6 +235,18 @@ struct Plan {
     r = std::min(d.d, d.dh);
     c = std::max(d.d, d.dh);
     mat3 = (size_t)3 * d.b * g.elems;
+    g.stacked = (muon && d.muon_stacked) ? 1 : 0;
+    if (g.stacked && S == 0) return fail("muon_stacked needs at least one Newton-Schulz iteration");
+    nsb.clear();
+    if (!g.stacked) {
+      nsb.push_back(NsBatch{3 * d.b, r, c, (g.tall(0) ? 1 : 0) | (g.tall(1) ? 2 : 0) | (g.tall(2) ? 4 : 0), d.b, 0, 0, 0});
+      sq_total = (size_t)3 * d.b * r * r;
+    } else {
+      const int rs = std::min(2 * d.dh, d.d), cs = std::max(2 * d.dh, d.d);
+      nsb.push_back(NsBatch{d.b, rs, cs, 2 * d.dh > d.d ? 1 : 0, d.b, 0, 0, 0});
+      nsb.push_back(NsBatch{d.b, r, c, g.tall(1) ? 1 : 0, d.b, d.b, (size_t)2 * d.b * g.elems, (size_t)d.b * rs * rs});
+      sq_total = (size_t)d.b * rs * rs + (size_t)d.b * r * r;
+    }
     nblk = std::max(1, std::min(256, (int)((g.elems + 2047) / 2048)));
     lr_slots = ceil_div(d.dh, 128) * 4;   // (hidden tiles) x (wave columns) of the widest update-backward tiling
     tiles = ceil_div(d.dh, TSA::BM) * ceil_div(d.d, TSA::BN);
@@ -244,7 +266,7 @@ struct Plan {
     s_g16 = muon ? sv.take((size_t)nupd * mat3 * nsz) : 0;
     s_norms = sv.take((size_t)std::max(1, nupd) * 3 * d.b * 4);
     s_xb = muon ? sv.take((size_t)nupd * std::max(1, S) * mat3 * nsz) : 0;
-    const size_t sq3 = (size_t)3 * d.b * r * r;
+    const size_t sq3 = sq_total;
     s_ab = muon ? sv.take((size_t)nupd * std::max(1, S) * sq3 * nsz) : 0;
     s_bb = muon ? sv.take((size_t)nupd * std::max(1, S) * sq3 * nsz) : 0;
     saved_bytes = sv.off + 256;
@@ -396,39 +418,48 @@ struct Runner {
     side = side_ctx();
     if (side && g_overlap) s_side = side->stream;
   }
-  // ---- fused Newton-Schulz: one launch per batch of at most 256 resident blocks
+  // ---- fused Newton-Schulz: launches of at most 256 resident blocks
   static bool tiles_fit(int r, int c, int edge) { return r % edge == 0 && c % edge == 0 && (r / edge) * (c / edge) <= 32; }
   // 192 x 192 tiles when the matrices fill at least half the chip with them, else 128 x 128 (more, smaller blocks)
-  bool ns_fused_small_tiles() const {
-    if (!tiles_fit(P.r, P.c, 128)) return false;
-    if (!tiles_fit(P.r, P.c, 192)) return true;
-    return 3 * d.b * (P.r / 192) * (P.c / 192) < 128;
+  static bool ns_fused_small_tiles(const NsBatch& B) {
+    if (!tiles_fit(B.r, B.c, 128)) return false;
+    if (!tiles_fit(B.r, B.c, 192)) return true;
+    return B.n * (B.r / 192) * (B.c / 192) < 128;
   }
-  bool ns_fused_ok() const {
+  bool ns_fused_ok(const NsBatch& B) const {
     if (!g_fused_ns || !side || !kNsBf16 || P.S < 1 || P.S > NS_FUSED_MAX_STEPS) return false;
-    return tiles_fit(P.r, P.c, 192) || tiles_fit(P.r, P.c, 128);
+    return tiles_fit(B.r, B.c, 192) || tiles_fit(B.r, B.c, 128);
+  }
+  bool ns_fused_any() const {
+    for (auto& B : P.nsb)
+      if (ns_fused_ok(B)) return true;
+    return false;
+  }
+  unsigned* ns_error_word() const { return scr<unsigned>(P.t_nssync) + (size_t)P.g.ns_count() * 32; }
+  // barrier lines and error word start at zero: once per Newton-Schulz phase, in front of its batches
+  void ns_clear_sync() {
+    const long long words = (long long)P.g.ns_count() * 32 + 32;
+    LACT_LAUNCH("k_fill_f32", "k_fill_f32", 0.0, k_fill_f32, dim3((unsigned)((words + 255) / 256)), dim3(256), s, scr<float>(P.t_nssync), 0.f, words);
   }
   template <class TS, bool BWD>
-  void launch_ns_fused_ts(NsFusedParams p) {
+  void launch_ns_fused_ts(NsFusedParams p, const NsBatch& B) {
     constexpr int SM = cmax(DmaSmem<TS, 1, row_stages<TS>()>::BYTES, StageTile<TS, 4>::BYTES);
     static bool once = (allow_big_lds(k_ns_fused<TS, BWD>, SM), true);
     (void)once;
-    const int total = 3 * d.b, nbm = (P.r / TS::BM) * (P.c / TS::BN);
+    const int nbm = (B.r / TS::BM) * (B.c / TS::BN);
     const int per = (256 / nbm) / 8 * 8;
-    unsigned* sync = scr<unsigned>(P.t_nssync);
-    const long long words = (long long)total * 32 + 32;
-    LACT_LAUNCH("k_fill_f32", "k_fill_f32", 0.0, k_fill_f32, dim3((unsigned)((words + 255) / 256)), dim3(256), s, reinterpret_cast<float*>(sync), 0.f, words);
-    p.r = P.r; p.c = P.c; p.S = P.S; p.nb = d.b; p.mask = tall_mask();
+    unsigned* sync = scr<unsigned>(P.t_nssync) + (size_t)B.first * 32;
+    p.r = B.r; p.c = B.c; p.S = P.S; p.nb = B.nb; p.mask = B.mask;
     for (int i = 0; i < 3 * P.S; ++i) p.coeffs[i] = P.coeffs[i];
-    p.error = sync + (size_t)total * 32;
+    p.error = ns_error_word();
     const double terms = BWD ? 6.0 : 3.0;
     static const std::string name = std::string("k_ns_fused<") + std::to_string(TS::BM) + "x" + std::to_string(TS::BN) + (BWD ? ",bwd>" : ",fwd>");
-    for (int z0 = 0; z0 < total; z0 += per) {
-      p.z0 = z0; p.n = std::min(per, total - z0); p.sync = sync + (size_t)z0 * 32;
+    for (int z0 = 0; z0 < B.n; z0 += per) {
+      p.z0 = z0; p.n = std::min(per, B.n - z0); p.sync = sync + (size_t)z0 * 32;
       const int grid = 8 * ((p.n + 7) / 8) * nbm;
       // fused launches of this process never overlap each other (each needs its groups resident as a whole)
       if (side->fused_recorded) (void)hipStreamWaitEvent(s, side->fused_done, 0);
-      LACT_LAUNCH_SMEM(name.c_str(), BWD ? "ns_bwd" : "ns_fwd", terms * 2.0 * P.r * P.r * P.c * P.S * p.n,
+      LACT_LAUNCH_SMEM(name.c_str(), BWD ? "ns_bwd" : "ns_fwd", terms * 2.0 * B.r * B.r * B.c * P.S * p.n,
                        (k_ns_fused<TS, BWD>), dim3(grid), dim3(DMA_THREADS), SM, s, p);
       if (!side->fused_done) (void)hipEventCreateWithFlags(&side->fused_done, hipEventDisableTiming);
       (void)hipEventRecord(side->fused_done, s);
@@ -436,9 +467,9 @@ struct Runner {
     }
   }
   template <bool BWD>
-  void launch_ns_fused(const NsFusedParams& p) {
-    if (ns_fused_small_tiles()) launch_ns_fused_ts<TS_SQ, BWD>(p);
-    else launch_ns_fused_ts<TS_NS, BWD>(p);
+  void launch_ns_fused(const NsFusedParams& p, const NsBatch& B) {
+    if (ns_fused_small_tiles(B)) launch_ns_fused_ts<TS_SQ, BWD>(p, B);
+    else launch_ns_fused_ts<TS_NS, BWD>(p, B);
   }
   // `waiter` waits for everything enqueued so far on `on`
   void wait_for(hipStream_t waiter, hipStream_t on) {
@@ -466,7 +497,7 @@ struct Runner {
   TN* g16(int u) const { return reinterpret_cast<TN*>(sv + P.s_g16) + (size_t)u * P.mat3; }
   float* norms(int u) const { return reinterpret_cast<float*>(sv + P.s_norms) + (size_t)u * 3 * d.b; }
   TN* xb(int u, int it) const { return reinterpret_cast<TN*>(sv + P.s_xb) + ((size_t)u * std::max(1, P.S) + it) * P.mat3; }
-  size_t sq3() const { return (size_t)3 * d.b * P.r * P.r; }
+  size_t sq3() const { return P.sq_total; }
   TN* ab(int u, int it) const { return reinterpret_cast<TN*>(sv + P.s_ab) + ((size_t)u * std::max(1, P.S) + it) * sq3(); }
   TN* bb(int u, int it) const { return reinterpret_cast<TN*>(sv + P.s_bb) + ((size_t)u * std::max(1, P.S) + it) * sq3(); }
   T* h(int i) const { return reinterpret_cast<T*>(sc + hsel[i]); }
@@ -504,7 +535,6 @@ struct Runner {
   }
   template <typename U> U* scr(size_t off) const { return reinterpret_cast<U*>(sc + off); }
 
-  int tall_mask() const { return (P.g.tall(0) ? 1 : 0) | (P.g.tall(1) ? 2 : 0) | (P.g.tall(2) ? 4 : 0); }
   long long hbs() const { return (long long)P.Tcap * d.dh; }
 
   HiddenParams hidden_params(int T_, const void* X, int ldx, long long bsx, const void* Y, int ldy, long long bsy, int ver) const {
@@ -594,6 +624,8 @@ struct Runner {
     p.cr = replace ? 1.f : 0.f;
     p.n0 = n0();
     p.weight_norm = d.weight_norm;
+    p.u_stacked = (P.muon && P.g.stacked) ? 1 : 0;
+    p.eps_in_sqrt = d.renorm_eps_in_sqrt ? 1 : 0;
     return p;
   }
 
@@ -688,30 +720,34 @@ struct Runner {
         p.xf = scr<float>(P.t_xf[0]); p.xb = xb(u, 0);
         p.u = P.S == 0 ? usave(u) : nullptr;
         p.plain_bf16 = d.ns_mode == LACT_NS_PLAIN_BF16;
-        LACT_LAUNCH("k_ns_scale", "k_ns_scale", 0.0, (k_ns_scale<TN>), dim3(P.nblk, 3 * d.b), dim3(256), s, p);
-        if (ns_fused_ok()) {
-          if constexpr (kNsBf16) {
-            NsFusedParams f;
-            memset(&f, 0, sizeof(f));
-            f.plain = d.ns_mode == LACT_NS_PLAIN_BF16;
-            f.xf[0] = scr<float>(P.t_xf[0]); f.xf[1] = scr<float>(P.t_xf[1]);
-            f.xb = xb(u, 0); f.xb_it_stride = (long long)P.mat3;
-            f.ab = ab(u, 0); f.bb = bb(u, 0); f.sq_it_stride = (long long)sq3();
-            f.xb_last = scr<uint16_t>(P.t_xbtmp); f.u_out = usave(u);
-            launch_ns_fused<false>(f);
+        LACT_LAUNCH("k_ns_scale", "k_ns_scale", 0.0, (k_ns_scale<TN>), dim3(P.nblk, P.g.ns_count()), dim3(256), s, p);
+        if (ns_fused_any()) ns_clear_sync();
+        for (const NsBatch& B : P.nsb) {
+          if (ns_fused_ok(B)) {
+            if constexpr (kNsBf16) {
+              NsFusedParams f;
+              memset(&f, 0, sizeof(f));
+              f.plain = d.ns_mode == LACT_NS_PLAIN_BF16;
+              f.xf[0] = scr<float>(P.t_xf[0]) + B.xoff; f.xf[1] = scr<float>(P.t_xf[1]) + B.xoff;
+              f.xb = xb(u, 0) + B.xoff; f.xb_it_stride = (long long)P.mat3;
+              f.ab = ab(u, 0) + B.sqoff; f.bb = bb(u, 0) + B.sqoff; f.sq_it_stride = (long long)sq3();
+              f.xb_last = scr<uint16_t>(P.t_xbtmp) + B.xoff; f.u_out = usave(u) + B.xoff;
+              launch_ns_fused<false>(f, B);
+            }
+            continue;
           }
-        } else
-        for (int it = 0; it < P.S; ++it) {
-          const bool last = it + 1 == P.S;
-          NsIter I;
-          I.n = 3 * d.b; I.r = P.r; I.c = P.c; I.nb_for_mask = d.b; I.mask = tall_mask(); I.plain = d.ns_mode == LACT_NS_PLAIN_BF16;
-          I.ca = P.coeffs[3 * it]; I.cb = P.coeffs[3 * it + 1]; I.cc = P.coeffs[3 * it + 2];
-          I.xf_in = scr<float>(P.t_xf[it & 1]); I.xb_in = xb(u, it);
-          I.ab = ab(u, it); I.bb = bb(u, it);
-          I.xf_out = last ? nullptr : scr<float>(P.t_xf[(it + 1) & 1]);
-          I.xb_out = last ? (void*)scr<TN>(P.t_xbtmp) : (void*)xb(u, it + 1);
-          I.u_out = last ? usave(u) : nullptr;
-          ns_iteration<TN>(I, s);
+          for (int it = 0; it < P.S; ++it) {
+            const bool last = it + 1 == P.S;
+            NsIter I;
+            I.n = B.n; I.r = B.r; I.c = B.c; I.nb_for_mask = B.nb; I.mask = B.mask; I.plain = d.ns_mode == LACT_NS_PLAIN_BF16;
+            I.ca = P.coeffs[3 * it]; I.cb = P.coeffs[3 * it + 1]; I.cc = P.coeffs[3 * it + 2];
+            I.xf_in = scr<float>(P.t_xf[it & 1]) + B.xoff; I.xb_in = xb(u, it) + B.xoff;
+            I.ab = ab(u, it) + B.sqoff; I.bb = bb(u, it) + B.sqoff;
+            I.xf_out = last ? nullptr : scr<float>(P.t_xf[(it + 1) & 1]) + B.xoff;
+            I.xb_out = last ? (void*)(scr<TN>(P.t_xbtmp) + B.xoff) : (void*)(xb(u, it + 1) + B.xoff);
+            I.u_out = last ? usave(u) + B.xoff : nullptr;
+            ns_iteration<TN>(I, s);
+          }
         }
       }
       {
@@ -721,7 +757,7 @@ struct Runner {
         p.wc_out = P.bf16 ? (void*)wc(ver + 1) : nullptr;
         if (u + 1 == P.nupd && w_out)
           for (int j = 0; j < 3; ++j) p.w_ext[j] = w_out[j];
-        if (P.muon && ns_fused_ok()) p.poison = scr<unsigned>(P.t_nssync) + (size_t)3 * d.b * 32;
+        if (P.muon && ns_fused_any()) p.poison = ns_error_word();
         LACT_LAUNCH("k_update_renorm", "k_update_renorm", 0.0, (k_update_renorm<T>), rowgrid, dim3(256), s, p);
       }
       ++ver;
@@ -943,57 +979,65 @@ struct Runner {
       }
       if (d.prenorm) carry_main = gw_idx;
       if (P.muon) {
-        const int n = 3 * d.b, r = P.r, c = P.c;
-        const long long xe = (long long)r * c, se = (long long)r * r;
-        TN* sg = scr<TN>(P.t_sg);
-        TN* gas = scr<TN>(P.t_gas);
-        if (ns_fused_ok()) {
-          if constexpr (kNsBf16) {
-            NsFusedParams f;
-            memset(&f, 0, sizeof(f));
-            f.xb = xb(u, 0); f.xb_it_stride = (long long)P.mat3;
-            f.ab = ab(u, 0); f.bb = bb(u, 0); f.sq_it_stride = (long long)sq3();
-            f.gxf[0] = scr<float>(P.t_gxf[0]); f.gxf[1] = scr<float>(P.t_gxf[1]);
-            f.gxb[0] = scr<uint16_t>(P.t_gxb[0]); f.gxb[1] = scr<uint16_t>(P.t_gxb[1]);
-            f.sg = reinterpret_cast<uint16_t*>(sg); f.gas = reinterpret_cast<uint16_t*>(gas);
-            launch_ns_fused<true>(f);
-            cur = P.S & 1;
+        if (ns_fused_any()) ns_clear_sync();
+        for (const NsBatch& B : P.nsb) {
+          const int n = B.n, r = B.r, c = B.c;
+          const long long xe = (long long)r * c, se = (long long)r * r;
+          TN* sg = scr<TN>(P.t_sg) + B.sqoff;
+          TN* gas = scr<TN>(P.t_gas) + B.sqoff;
+          if (ns_fused_ok(B)) {
+            if constexpr (kNsBf16) {
+              NsFusedParams f;
+              memset(&f, 0, sizeof(f));
+              f.xb = xb(u, 0) + B.xoff; f.xb_it_stride = (long long)P.mat3;
+              f.ab = ab(u, 0) + B.sqoff; f.bb = bb(u, 0) + B.sqoff; f.sq_it_stride = (long long)sq3();
+              f.gxf[0] = scr<float>(P.t_gxf[0]) + B.xoff; f.gxf[1] = scr<float>(P.t_gxf[1]) + B.xoff;
+              f.gxb[0] = scr<uint16_t>(P.t_gxb[0]) + B.xoff; f.gxb[1] = scr<uint16_t>(P.t_gxb[1]) + B.xoff;
+              f.sg = reinterpret_cast<uint16_t*>(sg); f.gas = reinterpret_cast<uint16_t*>(gas);
+              launch_ns_fused<true>(f, B);
+            }
+            continue;
           }
-        } else
-        for (int it = P.S - 1; it >= 0; --it) {
-          const float ca = P.coeffs[3 * it], cb = P.coeffs[3 * it + 1], cc = P.coeffs[3 * it + 2];
-          TN* gb = scr<TN>(P.t_gxb[cur]);
-          float* gf = scr<float>(P.t_gxf[cur]);
-          {  // Sg = G X^T + X G^T
-            auto p = row_params<2>();
-            set_term(p.t[0], gb, c, xe, xb(u, it), c, xe, c);
-            set_term(p.t[1], xb(u, it), c, xe, gb, c, xe, c);
-            p.M = r; p.N = r; p.out = sg; p.ldo = r; p.bso = se;
-            launch_row_gemm<TN, true, 2, EPI_STORE>("ns_bwd_sg", p, n, s);
+          int bc = 0;   // every batch starts from buffer 0 and ends in buffer S & 1
+          for (int it = P.S - 1; it >= 0; --it) {
+            const float ca = P.coeffs[3 * it], cb = P.coeffs[3 * it + 1], cc = P.coeffs[3 * it + 2];
+            TN* gb = scr<TN>(P.t_gxb[bc]) + B.xoff;
+            float* gf = scr<float>(P.t_gxf[bc]) + B.xoff;
+            TN* xk = xb(u, it) + B.xoff;
+            TN* ak = ab(u, it) + B.sqoff;
+            TN* bk = bb(u, it) + B.sqoff;
+            {  // Sg = G X^T + X G^T
+              auto p = row_params<2>();
+              set_term(p.t[0], gb, c, xe, xk, c, xe, c);
+              set_term(p.t[1], xk, c, xe, gb, c, xe, c);
+              p.M = r; p.N = r; p.out = sg; p.ldo = r; p.bso = se;
+              launch_row_gemm<TN, true, 2, EPI_STORE>("ns_bwd_sg", p, n, s);
+            }
+            {  // gA + gA^T = b Sg + c (Sg A + A Sg)
+              auto p = row_params<2>();
+              set_term(p.t[0], sg, r, se, ak, r, se, r);
+              set_term(p.t[1], ak, r, se, sg, r, se, r);
+              p.M = r; p.N = r; p.out = gas; p.ldo = r; p.bso = se;
+              p.aux = sg; p.ldaux = r; p.bsaux = se; p.alpha = cc; p.beta = cb;
+              launch_row_gemm<TN, true, 2, EPI_AXPBY>("ns_bwd_ga", p, n, s);
+            }
+            {  // gX = a G + B G + (gA + gA^T) X
+              auto p = row_params<2>();
+              set_term(p.t[0], bk, r, se, gb, c, xe, r);
+              set_term(p.t[1], gas, r, se, xk, c, xe, r);
+              p.M = r; p.N = c; p.ldo = c; p.bso = xe;
+              p.aux = gf; p.ldaux = c; p.bsaux = xe; p.alpha = 1.f; p.beta = ca;
+              p.out = scr<float>(P.t_gxf[bc ^ 1]) + B.xoff;
+              p.out_c = scr<TN>(P.t_gxb[bc ^ 1]) + B.xoff;
+              launch_row_gemm<TN, false, 2, EPI_AXPBY_F32_DUAL>("ns_bwd_gx", p, n, s);
+            }
+            bc ^= 1;
           }
-          {  // gA + gA^T = b Sg + c (Sg A + A Sg)
-            auto p = row_params<2>();
-            set_term(p.t[0], sg, r, se, ab(u, it), r, se, r);
-            set_term(p.t[1], ab(u, it), r, se, sg, r, se, r);
-            p.M = r; p.N = r; p.out = gas; p.ldo = r; p.bso = se;
-            p.aux = sg; p.ldaux = r; p.bsaux = se; p.alpha = cc; p.beta = cb;
-            launch_row_gemm<TN, true, 2, EPI_AXPBY>("ns_bwd_ga", p, n, s);
-          }
-          {  // gX = a G + B G + (gA + gA^T) X
-            auto p = row_params<2>();
-            set_term(p.t[0], bb(u, it), r, se, gb, c, xe, r);
-            set_term(p.t[1], gas, r, se, xb(u, it), c, xe, r);
-            p.M = r; p.N = c; p.ldo = c; p.bso = xe;
-            p.aux = gf; p.ldaux = c; p.bsaux = xe; p.alpha = 1.f; p.beta = ca;
-            p.out = scr<float>(P.t_gxf[cur ^ 1]);
-            p.out_c = scr<TN>(P.t_gxb[cur ^ 1]);
-            launch_row_gemm<TN, false, 2, EPI_AXPBY_F32_DUAL>("ns_bwd_gx", p, n, s);
-          }
-          cur ^= 1;
         }
+        cur = P.S & 1;
         NsDotParams dp;
         dp.g = P.g; dp.gx0 = scr<float>(P.t_gxf[cur]); dp.g16 = g16(u); dp.dot_part = scr<float>(P.t_dot);
-        LACT_LAUNCH("k_ns_bwd_dot", "k_ns_bwd_dot", 0.0, (k_ns_bwd_dot<TN>), dim3(P.nblk, 3 * d.b), dim3(256), s, dp);
+        LACT_LAUNCH("k_ns_bwd_dot", "k_ns_bwd_dot", 0.0, (k_ns_bwd_dot<TN>), dim3(P.nblk, P.g.ns_count()), dim3(256), s, dp);
       }
       {
         GradPrepParams p;
@@ -1007,7 +1051,7 @@ struct Runner {
         p.mbar = P.momentum ? mbar(u) : nullptr;
         p.gc = scr<T>(P.t_gc);
         p.mdot_part = scr<float>(P.t_mdot);
-        if (P.muon && ns_fused_ok()) p.poison = scr<unsigned>(P.t_nssync) + (size_t)3 * d.b * 32;
+        if (P.muon && ns_fused_any()) p.poison = ns_error_word();
         LACT_LAUNCH("k_grad_prep", "k_grad_prep", 0.0, (k_grad_prep<T, TN>), dim3(P.nblk, 3 * d.b), dim3(256), s, p);
         if (P.momentum) {
           gm_valid = true;
@@ -1103,7 +1147,7 @@ struct NsPlan {
   size_t o_g16, o_ss, o_norm, o_xf[2], o_xb[2], o_ab, o_bb, bytes;
   void build(int n, int rows, int cols) {
     // one "matrix kind" (index 0) of shape [rows, cols]: d = cols, dh = rows
-    g.d = cols; g.dh = rows; g.nb = n; g.elems = (long long)rows * cols;
+    g.d = cols; g.dh = rows; g.nb = n; g.elems = (long long)rows * cols; g.stacked = 0;
     r = std::min(rows, cols); c = std::max(rows, cols);
     nblk = std::max(1, std::min(256, (int)((g.elems + 2047) / 2048)));
     Bump b;

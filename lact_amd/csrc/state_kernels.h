@@ -13,16 +13,39 @@ namespace lact {
 struct MatGeom {
   int d, dh, nb;          // feature dim, hidden dim, batch*heads
   long long elems;        // d*dh
+  int stacked;            // Newton-Schulz runs on cat(dw0, dw2) [2dh, d] and on dw1 (fused-kernel variant) instead of three matrices
   __host__ __device__ int rows(int j) const { return j == 1 ? d : dh; }
   __host__ __device__ int cols(int j) const { return j == 1 ? dh : d; }
   __host__ __device__ bool tall(int j) const { return rows(j) > cols(j); }
   __host__ __device__ int maxrows() const { return d > dh ? d : dh; }
-  // index of original element e = i*cols + j inside the Newton-Schulz orientation
-  __device__ long long xidx(int j, long long e) const {
-    if (!tall(j)) return e;
-    const int c = cols(j), r = rows(j);
-    const long long i = e / c, k = e % c;
-    return k * r + i;
+  // ---- Newton-Schulz matrices.  They live in buffers of 3*nb*elems elements in "Newton-Schulz orientation"
+  // [r, c] = [min, max] (a matrix with more rows than columns is held transposed).  Unstacked: matrix z of the
+  // packed order at z*elems.  Stacked: nb matrices of 2*elems (w0 rows on top of w2 rows), then nb of elems (w1).
+  __host__ __device__ int ns_count() const { return stacked ? 2 * nb : 3 * nb; }
+  __host__ __device__ long long ns_elems(int m) const { return stacked && m < nb ? 2 * elems : elems; }
+  __host__ __device__ long long ns_base(int m) const { return stacked ? (m < nb ? m * 2 * elems : 2 * nb * elems + (m - nb) * elems) : m * elems; }
+  // Newton-Schulz matrix of packed matrix z = j*nb + ib
+  __host__ __device__ int ns_of(int z) const { return stacked ? (z / nb == 1 ? z : z % nb) : z; }
+  // packed matrices that make up Newton-Schulz matrix m: first and (stacked pair only) second
+  __host__ __device__ int ns_part0(int m) const { return m; }
+  __host__ __device__ int ns_part1(int m) const { return stacked && m < nb ? 2 * nb + m : -1; }
+  // rows of the matrix the orthogonalisation sees for kind j, and whether it is held transposed
+  __host__ __device__ int ns_rows(int j) const { return stacked && j != 1 ? 2 * dh : rows(j); }
+  __host__ __device__ bool ns_tall(int j) const { return ns_rows(j) > cols(j); }
+  // offset, inside its Newton-Schulz matrix, of element e = i*cols + k of packed matrix kind j
+  __host__ __device__ long long xidx(int j, long long e) const {
+    const int c = cols(j), nr = ns_rows(j);
+    const long long i = e / c + (stacked && j == 2 ? dh : 0), k = e % c;
+    return ns_tall(j) ? k * nr + i : i * c + k;
+  }
+  // four consecutive e map to four consecutive offsets
+  __host__ __device__ bool x_contiguous(int j) const { return !ns_tall(j); }
+  // offset of packed matrix z in the buffer that holds the orthogonalised update in original orientation
+  // (stacked: cat(U0, U2) per head, then U1)
+  __host__ __device__ long long u_off(int z) const {
+    if (!stacked) return z * elems;
+    const int j = z / nb, ib = z % nb;
+    return j == 0 ? ib * 2 * elems : (j == 2 ? (ib * 2 + 1) * elems : (2 * nb + ib) * elems);
   }
 };
 
@@ -102,7 +125,8 @@ __global__ void k_momentum_prep(const MomentumPrepParams p) {
   const float mb = (p.m_prev && p.mbar) ? p.mbar[ib] : 0.f;
   const size_t zo = (size_t)z * p.g.elems, stride = (size_t)3 * p.g.nb * p.g.elems;
   float* ext = p.m_ext[j] ? p.m_ext[j] + (size_t)ib * p.g.elems : nullptr;
-  const bool tall = p.g.tall(j);
+  const bool contiguous = p.g.x_contiguous(j);
+  const size_t xo = p.g.ns_base(p.g.ns_of(z));
   float ss = 0.f;
   for (long long e = R.e0 + threadIdx.x * 4; e < R.e1; e += blockDim.x * 4) {
     float4 v = ld4(p.partial + zo + e);
@@ -119,9 +143,9 @@ __global__ void k_momentum_prep(const MomentumPrepParams p) {
     if (ext) st4(ext + e, v);
     if (p.g16) {
       const float4 f = f4(Elem<TN>::rnd(v.x), Elem<TN>::rnd(v.y), Elem<TN>::rnd(v.z), Elem<TN>::rnd(v.w));
-      TN* g = reinterpret_cast<TN*>(p.g16) + zo;
-      if (!tall) {
-        Elem<TN>::store4(g + e, f.x, f.y, f.z, f.w);
+      TN* g = reinterpret_cast<TN*>(p.g16) + xo;
+      if (contiguous) {
+        Elem<TN>::store4(g + p.g.xidx(j, e), f.x, f.y, f.z, f.w);
       } else {
         Elem<TN>::store(g + p.g.xidx(j, e), f.x); Elem<TN>::store(g + p.g.xidx(j, e + 1), f.y);
         Elem<TN>::store(g + p.g.xidx(j, e + 2), f.z); Elem<TN>::store(g + p.g.xidx(j, e + 3), f.w);
@@ -144,21 +168,25 @@ struct NsScaleParams {
   float* u;              // [3b][elems] original orientation, or null (only when zero iterations follow)
   int plain_bf16;        // reference without autocast: norm and quotient are bf16 tensors
 };
+// Grid (chunks, Newton-Schulz matrices).  ss_part is indexed by packed matrix.
 template <typename TN>
 __global__ void k_ns_scale(const NsScaleParams p) {
-  const int z = blockIdx.y, j = z / p.g.nb;
+  const int m = blockIdx.y;
   float ss = 0.f;
-  for (int i = 0; i < p.nparts; ++i) ss += p.ss_part[(size_t)z * p.nparts + i];
+  for (int i = 0; i < p.nparts; ++i) ss += p.ss_part[(size_t)p.g.ns_part0(m) * p.nparts + i];
+  if (p.g.ns_part1(m) >= 0)
+    for (int i = 0; i < p.nparts; ++i) ss += p.ss_part[(size_t)p.g.ns_part1(m) * p.nparts + i];
   float n = sqrtf(ss);
   if (p.plain_bf16) n = round_bf16(n);
-  if (blockIdx.x == 0 && threadIdx.x == 0) p.norms[z] = n;
+  if (blockIdx.x == 0 && threadIdx.x == 0) p.norms[m] = n;
   float den = n + 1e-7f;
   if (p.plain_bf16) den = round_bf16(den);
   const float inv = 1.f / den;
-  const FlatRange R(p.g.elems);
-  const size_t zo = (size_t)z * p.g.elems;
+  const FlatRange R(p.g.ns_elems(m));
+  const size_t zo = p.g.ns_base(m);
+  // `u` (only when zero iterations follow; never stacked): original orientation of matrix m = packed z
+  const int j = m / p.g.nb;
   const bool tall = p.g.tall(j);
-  // walks the Newton-Schulz orientation x; the original-orientation copy `u` is the scattered one when tall
   for (long long x = R.e0 + threadIdx.x * 4; x < R.e1; x += blockDim.x * 4) {
     float v[4];
     Elem<TN>::load4(reinterpret_cast<const TN*>(p.g16) + zo + x, v);
@@ -189,6 +217,8 @@ struct RenormParams {
   const float* raw; float cr;      // raw gradient added on top (bidirectional layer), or null
   const float* n0;
   int weight_norm;
+  int u_stacked;                   // `u` is laid out per Newton-Schulz matrix (MatGeom::u_off), not packed
+  int eps_in_sqrt;                 // y = w_hat / sqrt(|w_hat|^2 + eps) * n0 (fused-kernel variant) instead of / (|w_hat| + eps)
   float* main_out;                 // un-normalised accumulator (pre-norm) or null
   float* wf_out; void* wc_out;     // new weights: fp32 state and compute-type copy (may be null)
   float* w_ext[3];                 // caller's weight outputs [b][elems] (same values as wf_out), each nullable
@@ -201,8 +231,9 @@ struct RenormParams {
   float* gn0;                      // [3b][maxrows], accumulated
   float* gxf; void* gxb;           // the same gradient in Newton-Schulz orientation (fp32 + Newton-Schulz type) or null
 };
-__device__ __forceinline__ float4 renorm_w_hat4(const RenormParams& p, size_t off) {
-  float4 v = ld4(p.u + off);
+// off: offset in the packed arrays; uo: offset of the same element in `u`
+__device__ __forceinline__ float4 renorm_w_hat4(const RenormParams& p, size_t off, size_t uo) {
+  float4 v = ld4(p.u + uo);
   if (p.cw != 0.f) {
     const float4 b = ld4(p.base + off);
     v.x += p.cw * b.x; v.y += p.cw * b.y; v.z += p.cw * b.z; v.w += p.cw * b.w;
@@ -229,6 +260,7 @@ __global__ void k_update_renorm(const RenormParams p) {
   if (row >= p.g.rows(j)) return;
   const int cols = p.g.cols(j);
   const size_t o = (size_t)z * p.g.elems + (size_t)row * cols;
+  const size_t uo = (p.u_stacked ? (size_t)p.g.u_off(z) : (size_t)z * p.g.elems) + (size_t)row * cols;
   float* ext = p.w_ext[j] ? p.w_ext[j] + (size_t)ib * p.g.elems + (size_t)row * cols : nullptr;
   const bool keep = cols <= 256 * ROW_VEC_MAX;
   float4 vv[ROW_VEC_MAX];
@@ -237,16 +269,16 @@ __global__ void k_update_renorm(const RenormParams p) {
   for (int i = 0; i < ROW_VEC_MAX; ++i) {
     const int c = lane * 4 + i * 256;
     if (c < cols) {
-      vv[i] = renorm_w_hat4(p, o + c);
+      vv[i] = renorm_w_hat4(p, o + c, uo + c);
       ss += dot4(vv[i], vv[i]);
     }
   }
   for (int c = lane * 4 + ROW_VEC_MAX * 256; c < cols; c += 256) {
-    const float4 v = renorm_w_hat4(p, o + c);
+    const float4 v = renorm_w_hat4(p, o + c, uo + c);
     ss += dot4(v, v);
   }
   ss = wave_sum(ss);
-  float den = sqrtf(ss) + 1e-5f;
+  float den = p.eps_in_sqrt ? sqrtf(ss + 1e-5f) : sqrtf(ss) + 1e-5f;
   if (p.poison && *p.poison) den = __uint_as_float(0x7fc00000u);
   const float n0 = p.weight_norm ? p.n0[(size_t)z * p.g.maxrows() + row] : 1.f;
   auto emit = [&](int c, const float4& v) {
@@ -264,7 +296,7 @@ __global__ void k_update_renorm(const RenormParams p) {
     if (c < cols) emit(c, vv[i]);
   }
   if (!keep)
-    for (int c = lane * 4 + ROW_VEC_MAX * 256; c < cols; c += 256) emit(c, renorm_w_hat4(p, o + c));
+    for (int c = lane * 4 + ROW_VEC_MAX * 256; c < cols; c += 256) emit(c, renorm_w_hat4(p, o + c, uo + c));
 }
 
 // backward of the line above.  y = w_hat*n0/(r+eps), r = ||w_hat||:
@@ -274,29 +306,39 @@ __global__ void k_renorm_bwd(const RenormParams p) {
   const int z = blockIdx.y, j = z / p.g.nb;
   const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (row >= p.g.rows(j)) return;
-  const int cols = p.g.cols(j), rows = p.g.rows(j);
-  const size_t zo = (size_t)z * p.g.elems, o = zo + (size_t)row * cols;
-  const bool tall = p.g.tall(j);
+  const int cols = p.g.cols(j);
+  const size_t o = (size_t)z * p.g.elems + (size_t)row * cols;
+  const size_t uo = (p.u_stacked ? (size_t)p.g.u_off(z) : (size_t)z * p.g.elems) + (size_t)row * cols;
+  const size_t xo = p.g.ns_base(p.g.ns_of(z));
+  const bool contiguous = p.g.x_contiguous(j);
   float c0 = 1.f, c1 = 0.f;
   if (p.weight_norm) {
     float ss = 0.f, dot = 0.f;
     for (int c = lane * 4; c < cols; c += 256) {
-      const float4 v = renorm_w_hat4(p, o + c);
+      const float4 v = renorm_w_hat4(p, o + c, uo + c);
       ss += dot4(v, v);
       if (p.gy || p.gy2) dot += dot4(v, renorm_gy4(p, o + c));
     }
     ss = wave_sum(ss);
     dot = wave_sum(dot);
-    const float r = sqrtf(ss), n0 = p.n0[(size_t)z * p.g.maxrows() + row];
-    c0 = n0 / (r + 1e-5f);
-    c1 = r > 0.f ? dot * n0 / (r * (r + 1e-5f) * (r + 1e-5f)) : 0.f;
-    if (lane == 0) p.gn0[(size_t)z * p.g.maxrows() + row] += dot / (r + 1e-5f);
+    const float n0 = p.n0[(size_t)z * p.g.maxrows() + row];
+    if (p.eps_in_sqrt) {   // den = sqrt(r^2 + eps):  d den / d w = w / den
+      const float den = sqrtf(ss + 1e-5f);
+      c0 = n0 / den;
+      c1 = dot * n0 / (den * den * den);
+      if (lane == 0) p.gn0[(size_t)z * p.g.maxrows() + row] += dot / den;
+    } else {               // den = r + eps:  d den / d w = w / r
+      const float r = sqrtf(ss);
+      c0 = n0 / (r + 1e-5f);
+      c1 = r > 0.f ? dot * n0 / (r * (r + 1e-5f) * (r + 1e-5f)) : 0.f;
+      if (lane == 0) p.gn0[(size_t)z * p.g.maxrows() + row] += dot / (r + 1e-5f);
+    }
   }
   for (int c = lane * 4; c < cols; c += 256) {
     float4 gv = renorm_gy4(p, o + c);
     gv = f4(gv.x * c0, gv.y * c0, gv.z * c0, gv.w * c0);
     if (p.weight_norm) {
-      const float4 w = renorm_w_hat4(p, o + c);
+      const float4 w = renorm_w_hat4(p, o + c, uo + c);
       gv.x -= w.x * c1; gv.y -= w.y * c1; gv.z -= w.z * c1; gv.w -= w.w * c1;
     }
     if (p.carry_in) {
@@ -304,15 +346,17 @@ __global__ void k_renorm_bwd(const RenormParams p) {
       gv.x += ci.x; gv.y += ci.y; gv.z += ci.z; gv.w += ci.w;
     }
     st4(p.gw_hat + o + c, gv);
-    if (p.gxf) {
-      if (!tall) {
-        st4(p.gxf + o + c, gv);
-        Elem<TN>::store4(reinterpret_cast<TN*>(p.gxb) + o + c, gv.x, gv.y, gv.z, gv.w);
-      } else {   // element (row, c) sits at c*rows + row in the Newton-Schulz orientation
+    if (p.gxf) {   // the same gradient where Newton-Schulz holds this matrix
+      const long long e = (long long)row * cols + c;
+      if (contiguous) {
+        const size_t x = xo + p.g.xidx(j, e);
+        st4(p.gxf + x, gv);
+        Elem<TN>::store4(reinterpret_cast<TN*>(p.gxb) + x, gv.x, gv.y, gv.z, gv.w);
+      } else {
         const float g[4] = {gv.x, gv.y, gv.z, gv.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const size_t x = zo + (size_t)(c + i) * rows + row;
+          const size_t x = xo + p.g.xidx(j, e + i);
           p.gxf[x] = g[i];
           Elem<TN>::store(reinterpret_cast<TN*>(p.gxb) + x, g[i]);
         }
@@ -326,12 +370,13 @@ struct NsDotParams {
   MatGeom g;
   const float* gx0; const void* g16; float* dot_part;
 };
+// Grid (chunks, Newton-Schulz matrices): <gradient at X0, Newton-Schulz input> per matrix.
 template <typename TN>
 __global__ void k_ns_bwd_dot(const NsDotParams p) {
   __shared__ float red[16];
-  const int z = blockIdx.y;
-  const FlatRange R(p.g.elems);
-  const size_t zo = (size_t)z * p.g.elems;
+  const int m = blockIdx.y;
+  const FlatRange R(p.g.ns_elems(m));
+  const size_t zo = p.g.ns_base(m);
   float s = 0.f;
   for (long long e = R.e0 + threadIdx.x * 4; e < R.e1; e += blockDim.x * 4) {
     float g[4];
@@ -339,7 +384,7 @@ __global__ void k_ns_bwd_dot(const NsDotParams p) {
     s += dot4(ld4(p.gx0 + zo + e), f4(g[0], g[1], g[2], g[3]));
   }
   s = block_sum(s, red);
-  if (threadIdx.x == 0) p.dot_part[(size_t)z * gridDim.x + blockIdx.x] = s;
+  if (threadIdx.x == 0) p.dot_part[(size_t)m * gridDim.x + blockIdx.x] = s;
 }
 
 struct GradPrepParams {
@@ -359,9 +404,10 @@ __global__ void k_grad_prep(const GradPrepParams p) {
   const int z = blockIdx.y, j = z / p.g.nb, ib = z % p.g.nb;
   float c0 = 1.f, c1 = 0.f;
   if (p.muon) {
+    const int m = p.g.ns_of(z);
     float dot = 0.f;
-    for (int i = 0; i < p.nparts; ++i) dot += p.dot_part[(size_t)z * p.nparts + i];
-    const float n = p.norms[z];
+    for (int i = 0; i < p.nparts; ++i) dot += p.dot_part[(size_t)m * p.nparts + i];
+    const float n = p.norms[m];
     c0 = 1.f / (n + 1e-7f);
     c1 = n > 0.f ? dot / (n * (n + 1e-7f) * (n + 1e-7f)) : 0.f;
     if (p.poison && *p.poison) c0 = __uint_as_float(0x7fc00000u);
@@ -369,7 +415,8 @@ __global__ void k_grad_prep(const GradPrepParams p) {
   const float mb = p.mbar ? p.mbar[ib] : 0.f;
   const FlatRange R(p.g.elems);
   const size_t zo = (size_t)z * p.g.elems;
-  const bool tall = p.g.tall(j);
+  const size_t xo = p.g.ns_base(p.g.ns_of(z));
+  const bool contiguous = p.g.x_contiguous(j);
   float md = 0.f;
   for (long long e = R.e0 + threadIdx.x * 4; e < R.e1; e += blockDim.x * 4) {
     const size_t o = zo + e;
@@ -377,14 +424,15 @@ __global__ void k_grad_prep(const GradPrepParams p) {
     if (p.muon) {
       float4 gx;
       float g[4];
-      if (!tall) {
-        gx = ld4(p.gx0 + o);
-        Elem<TN>::load4(reinterpret_cast<const TN*>(p.g16) + o, g);
+      if (contiguous) {
+        const size_t x = xo + p.g.xidx(j, e);
+        gx = ld4(p.gx0 + x);
+        Elem<TN>::load4(reinterpret_cast<const TN*>(p.g16) + x, g);
       } else {
         float t[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const size_t x = zo + p.g.xidx(j, e + i);
+          const size_t x = xo + p.g.xidx(j, e + i);
           t[i] = p.gx0[x];
           g[i] = Elem<TN>::load(reinterpret_cast<const TN*>(p.g16) + x);
         }

@@ -38,6 +38,10 @@ class Program:
     detach_norms: bool = False
     muon_replaces_weight: bool = False
     ns_mode: int = 0   # 0: bf16 GEMMs + fp32 iterate (autocast), 1: bf16 iterate (no autocast), 2: fp32 (exact)
+    # fused-kernel variant (lact_llm/lact_model/ttt_operation_fused_kernel.py): Newton-Schulz on the stacked
+    # gradient cat(dw0, dw2); eps inside the sqrt of the row renorm
+    muon_stacked: bool = False
+    renorm_eps_in_sqrt: bool = False
 
     @property
     def n_updates(self) -> int:
@@ -103,6 +107,7 @@ class _Call:
         D.prenorm, D.weight_norm = int(prog.prenorm), int(prog.weight_norm)
         D.detach_norms, D.muon_replaces_weight = int(prog.detach_norms), int(prog.muon_replaces_weight)
         D.ns_mode = int(prog.ns_mode)
+        D.muon_stacked, D.renorm_eps_in_sqrt = int(prog.muon_stacked), int(prog.renorm_eps_in_sqrt)
         D.q_bs, D.q_ld = q.stride(0), q.stride(1)
         if k is not None:
             D.k_bs, D.k_ld, D.v_bs, D.v_ld = k.stride(0), k.stride(1), v.stride(0), v.stride(1)

@@ -26,10 +26,12 @@ def zeropower_via_newtonschulz5(G: torch.Tensor) -> torch.Tensor:
     return ops.newton_schulz(G, NS5_COEFFS, ns_mode=ops.NS_AUTOCAST if torch.is_autocast_enabled() else ops.NS_PLAIN_BF16)
 
 
-def _block_causal(w0, w1, w2, q, k, v, lr0, lr1, lr2, chunk_size, use_muon, momentum, prenorm):
+def _block_causal(w0, w1, w2, q, k, v, lr0, lr1, lr2, chunk_size, use_muon, momentum, prenorm,
+                  muon_stacked=False, renorm_eps_in_sqrt=False):
     prog = Program(steps=block_causal_steps(k.shape[1], chunk_size), out_len=q.shape[1],
                    ns_coeffs=NS5_COEFFS if use_muon else None, prenorm=prenorm,
-                   ns_mode=ops._ns_mode(q))
+                   ns_mode=ops._ns_mode(q), muon_stacked=muon_stacked and use_muon,
+                   renorm_eps_in_sqrt=renorm_eps_in_sqrt)
     out, _, _ = run_program(prog, w0, w1, w2, q, k, v, lr0, lr1, lr2, momentum)
     return out
 
@@ -48,3 +50,25 @@ def prenorm_block_causal_lact_swiglu(w0: torch.Tensor, w1: torch.Tensor, w2: tor
                                      momentum: Optional[torch.Tensor] = None) -> torch.Tensor:
     """ttt_operation.py:219-364."""
     return _block_causal(w0, w1, w2, q, k, v, lr0, lr1, lr2, chunk_size, use_muon, momentum, True)
+
+
+def postnorm_block_causal_lact_swiglu_fused_kernel_triton(w0: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
+                                                          q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                                                          lr0: torch.Tensor, lr1: torch.Tensor, lr2: torch.Tensor,
+                                                          chunk_size: int = 2048, use_muon: bool = False,
+                                                          momentum: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """ttt_operation_fused_kernel.py:67-199 (the layer's `use_fused_kernel=True` path, layer_lact_swiglu.py:525-528):
+    same schedule as block_causal_lact_swiglu; Muon orthogonalises cat(dw0, dw2) as one [2dh, d] matrix and the
+    row renorm has eps inside the sqrt."""
+    return _block_causal(w0, w1, w2, q, k, v, lr0, lr1, lr2, chunk_size, use_muon, momentum, False,
+                         muon_stacked=True, renorm_eps_in_sqrt=True)
+
+
+def prenorm_block_causal_lact_swiglu_fused_kernel_triton(w0: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
+                                                         q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                                                         lr0: torch.Tensor, lr1: torch.Tensor, lr2: torch.Tensor,
+                                                         chunk_size: int = 2048, use_muon: bool = False,
+                                                         momentum: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """ttt_operation_fused_kernel.py:202-338 (layer_lact_swiglu.py:493-496): pre-norm accumulator, stacked Muon,
+    eps outside the sqrt (:322-327)."""
+    return _block_causal(w0, w1, w2, q, k, v, lr0, lr1, lr2, chunk_size, use_muon, momentum, True, muon_stacked=True)

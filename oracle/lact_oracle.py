@@ -170,8 +170,14 @@ def fast_weight_grads(w0, w1, w2, k, v, lr0, lr1, lr2, num: Numerics = Numerics(
     return dw0, dw1, dw2
 
 
-def renorm(w: torch.Tensor, w_norm0: torch.Tensor, num: Numerics = Numerics()) -> torch.Tensor:
-    """ttt_operation.py:198-200: rows rescaled to their initial L2 norm, eps outside the sqrt."""
+def renorm(w: torch.Tensor, w_norm0: torch.Tensor, num: Numerics = Numerics(), eps_in_sqrt: bool = False) -> torch.Tensor:
+    """ttt_operation.py:198-200: rows rescaled to their initial L2 norm, eps outside the sqrt.
+    eps_in_sqrt: the fused variant's kernel (l2norm_triton_kernels.py:205-214, "eps is inside the sqrt"):
+    y = x / sqrt(sum(x^2) + eps) * scale, statistics in fp32."""
+    if eps_in_sqrt:
+        wf = w.float()
+        rstd = torch.rsqrt((wf * wf).sum(dim=2, keepdim=True) + 1e-5)
+        return (wf * rstd * w_norm0.float()).to(w.dtype)
     return w / (num.norm(w, dim=2) + 1e-5) * w_norm0
 
 
@@ -188,12 +194,17 @@ def run_program(w0, w1, w2, q, k, v, lr0, lr1, lr2, steps: Sequence[Step], *,
                 muon_replaces_weight: bool = False,
                 cast_lr_operand: bool = True,
                 out_rows: Optional[int] = None,
-                scatter_output: bool = True):
+                scatter_output: bool = True,
+                stack_muon: bool = False,
+                eps_in_sqrt: bool = False):
     """Runs UPDATE / APPLY steps over one sequence.  LLM layout: w0,w2 [b,dh,dk], w1 [b,dv,dh].
 
     ns_coeffs=None means no Muon.  `muon_replaces_weight` is the bidirectional layer's behaviour
     (bidirectional_lact_layer.py:139-146): the orthogonalised gradient overwrites the weight and
     the raw gradient is then added, w_hat = NS(dw) + dw.
+    `stack_muon` / `eps_in_sqrt` are the two places where the fused-kernel driver differs in semantics
+    (ttt_operation_fused_kernel.py:106,168-173): Newton-Schulz runs on the stacked gradient cat(dw0, dw2)
+    [b, 2dh, d] (one Frobenius norm, one orthogonalisation) and the row renorm has eps inside the sqrt.
     Returns (output, (w0, w1, w2), (m0, m1, m2) or None).
     """
     def init_norm(w):
@@ -220,7 +231,11 @@ def run_program(w0, w1, w2, q, k, v, lr0, lr1, lr2, steps: Sequence[Step], *,
             dw2 = dw2 + mom[2] * m
             mom = [dw0, dw1, dw2]
         raw = (dw0, dw1, dw2)
-        if ns_coeffs is not None:                   # ttt_operation.py:181-184
+        if ns_coeffs is not None and stack_muon:    # ttt_operation_fused_kernel.py:168-170
+            dw1 = newton_schulz(dw1, ns_coeffs, num)
+            stacked = newton_schulz(torch.cat([dw0, dw2], dim=1), ns_coeffs, num)
+            dw0, dw2 = stacked[:, :dw0.shape[1]], stacked[:, dw0.shape[1]:]
+        elif ns_coeffs is not None:                 # ttt_operation.py:181-184
             dw1 = newton_schulz(dw1, ns_coeffs, num)
             dw0 = newton_schulz(dw0, ns_coeffs, num)
             dw2 = newton_schulz(dw2, ns_coeffs, num)
@@ -230,7 +245,8 @@ def run_program(w0, w1, w2, q, k, v, lr0, lr1, lr2, steps: Sequence[Step], *,
             base = (main0, main1, main2) if prenorm else (w0, w1, w2)
             main0, main1, main2 = base[0] + dw0, base[1] + dw1, base[2] + dw2
         if weight_norm:                             # ttt_operation.py:198-200 / :348-350
-            w0, w1, w2 = renorm(main0, n0, num), renorm(main1, n1, num), renorm(main2, n2, num)
+            w0, w1, w2 = (renorm(main0, n0, num, eps_in_sqrt), renorm(main1, n1, num, eps_in_sqrt),
+                          renorm(main2, n2, num, eps_in_sqrt))
         else:
             w0, w1, w2 = main0, main1, main2
 
@@ -309,6 +325,30 @@ def prenorm_block_causal_lact_swiglu(w0, w1, w2, q, k, v, lr0, lr1, lr2, chunk_s
     """ttt_operation.py:219-364."""
     return block_causal_lact_swiglu(w0, w1, w2, q, k, v, lr0, lr1, lr2, chunk_size, use_muon,
                                     momentum, num=num, prenorm=True)
+
+
+def postnorm_block_causal_lact_swiglu_fused_kernel_triton(w0, w1, w2, q, k, v, lr0, lr1, lr2, chunk_size: int = 2048,
+                                                          use_muon: bool = False, momentum=None, *,
+                                                          num: Numerics = Numerics()):
+    """ttt_operation_fused_kernel.py:67-199: the schedule of block_causal_lact_swiglu (padding to whole chunks
+    changes nothing: only whole chunks update), Muon on the stacked cat(dw0, dw2), eps inside the sqrt."""
+    out, _, _ = run_program(w0, w1, w2, q, k, v, lr0, lr1, lr2,
+                            block_causal_steps(k.shape[1], chunk_size), num=num,
+                            ns_coeffs=NS5_COEFFS if use_muon else None, momentum=momentum,
+                            stack_muon=True, eps_in_sqrt=True)
+    return out
+
+
+def prenorm_block_causal_lact_swiglu_fused_kernel_triton(w0, w1, w2, q, k, v, lr0, lr1, lr2, chunk_size: int = 2048,
+                                                         use_muon: bool = False, momentum=None, *,
+                                                         num: Numerics = Numerics()):
+    """ttt_operation_fused_kernel.py:202-338: pre-norm accumulator, Muon on the stacked gradient, eps outside
+    the sqrt (:322-327)."""
+    out, _, _ = run_program(w0, w1, w2, q, k, v, lr0, lr1, lr2,
+                            block_causal_steps(k.shape[1], chunk_size), num=num,
+                            ns_coeffs=NS5_COEFFS if use_muon else None, momentum=momentum, prenorm=True,
+                            stack_muon=True)
+    return out
 
 
 def block_causal_lact_swiglu_minimal(w0, w1, w2, q, k, v, lr0, lr1, lr2, momentum=None,

@@ -510,3 +510,61 @@ def test_fused_newton_schulz_is_bit_identical(b, d, dh):
         assert torch.equal(o1, o0)
         for n in g0:
             assert torch.equal(g1[n], g0[n]), n
+
+
+# ---- fused-kernel variant (ttt_operation_fused_kernel.py): stacked Muon, eps inside the sqrt -------------
+def fused_variant_pair(C, use_muon, prenorm):
+    hf = T.prenorm_block_causal_lact_swiglu_fused_kernel_triton if prenorm else T.postnorm_block_causal_lact_swiglu_fused_kernel_triton
+    of = O.prenorm_block_causal_lact_swiglu_fused_kernel_triton if prenorm else O.postnorm_block_causal_lact_swiglu_fused_kernel_triton
+    return (lambda t: hf(*args9(t), C, use_muon, t["momentum"]),
+            lambda t, num: of(*args9(t), C, use_muon, t["momentum"], num=num))
+
+
+@pytest.mark.parametrize("b,L,d,dh,C,prenorm", [
+    (2, 3 * 64 + 5, 64, 64, 64, False),       # stacked [128, 64]: held transposed
+    (2, 2 * 96 + 17, 128, 64, 96, True),      # stacked [128, 128]: square; w1 [128, 64] transposed
+    (2, 2 * 64 + 9, 256, 64, 64, False),      # stacked [128, 256]: as it lies
+    (2, 3 * 128, 384, 384, 128, False)])      # 760M shape: stacked [768, 384] -> fused kernel on [384, 768]
+def test_fused_variant_exact_arithmetic(b, L, d, dh, C, prenorm):
+    """fp32 activations + fp32 Newton-Schulz against the float64 oracle: pins the stacked orthogonalisation
+    (forward and backward, every layout case) and the eps-inside-sqrt renorm with its backward."""
+    say("fused variant exact", b, L, d, dh, C, prenorm)
+    inp = problem(b, L, d, dh, 19, torch.float32, momentum=True, lr_shift=-1.0)
+    hip, orc = fused_variant_pair(C, True, prenorm)
+    g = clone_to(inp, DEV)
+    with ops.newton_schulz_mode(ops.NS_FP32):
+        out = hip(g)
+    go = torch.randn(out.shape, generator=torch.Generator().manual_seed(3))
+    res = {"out": out, **grads_of(out, g, go.to(DEV))}
+    c64 = clone_to(inp, "cpu", dtype_map=lambda t: torch.float64)
+    o64 = orc(c64, EXACT)
+    ref = {"out": o64, **grads_of(o64, c64, go.double())}
+    errs = compare(res, ref)
+    say("  ", errs)
+    assert max(errs.values()) < 1e-3
+
+
+def test_fused_variant_small_rows_separate_the_eps_conventions():
+    """Weights with tiny rows (|row|^2 ~ eps): the two renorm conventions differ by tens of percent there, so
+    agreement with the oracle at 1e-3 shows the kernel has eps where the fused variant has it."""
+    say("fused variant tiny rows")
+    b, L, d, dh, C = 2, 2 * 64 + 3, 64, 64, 64
+    inp = problem(b, L, d, dh, 23, torch.float32, momentum=False, lr_shift=-9.0)
+    for n in ("w0", "w1", "w2"):
+        inp[n] = inp[n] * 3e-3
+    hip, orc = fused_variant_pair(C, False, False)
+    res, ref = run_both(hip, orc, inp, PLAIN)
+    errs = compare(res, ref)
+    say("  ", errs)
+    assert max(errs.values()) < 1e-3
+    other = O.block_causal_lact_swiglu(*args9(clone_to(inp, "cpu", grad=False)), C, False, None, num=PLAIN)
+    assert O.rel_l2(ref["out"][:, C:], other[:, C:]) > 0.02
+
+
+@pytest.mark.parametrize("b,L,d,dh,C,prenorm", [(2, 3 * 64 + 5, 64, 64, 64, False), (4, 1024, 384, 384, 512, False),
+                                                (3, 3 * 256, 128, 256, 256, True)])
+def test_fused_variant_bf16_muon(b, L, d, dh, C, prenorm):
+    say("fused variant bf16 muon", b, L, d, dh, C, prenorm)
+    inp = problem(b, L, d, dh, 29, torch.bfloat16, momentum=True)
+    res, ref, r64 = run_both(*fused_variant_pair(C, True, prenorm), inp, AC, ref64=True)
+    assert_within_noise_floor(res, ref, r64, "fused-variant")

@@ -292,3 +292,58 @@ def test_whole_op_gradcheck_fp64():
     args = [t.clone().requires_grad_(True) for t in (w0, w1, w2, q, k, v, lr0, lr1, lr2, mom)]
     fn = lambda *a: O.block_causal_lact_swiglu(*a[:9], 8, True, a[9], num=F64)
     assert torch.autograd.gradcheck(fn, args, eps=1e-6, atol=1e-5, rtol=1e-4)
+
+
+# ---- fused-kernel variant (ttt_operation_fused_kernel.py) -----------------------------------------
+def test_fused_variant_orthogonalises_the_stacked_gradient():
+    """One update, no renorm, exact arithmetic: cat(w0', w2') - cat(w0, w2) must be the quintic acting on the
+    singular values of the STACKED gradient cat(dw0, dw2) / ||.||_F (one SVD of the [2dh, d] matrix), and
+    w1' - w1 the same for dw1 alone.  Orthogonalising dw0 and dw2 separately fails this."""
+    w0, w1, w2, q, k, v, lr0, lr1, lr2 = rand_problem(b=2, L=24, d=6, dh=5)
+    L = k.shape[1]
+    steps = [O.Step(O.UPDATE, 0, L), O.Step(O.APPLY, 0, L)]
+    _, (n0, n1, n2), _ = O.run_program(w0, w1, w2, q, k, v, lr0, lr1, lr2, steps, num=F64, ns_coeffs=O.NS5_COEFFS,
+                                      weight_norm=False, stack_muon=True)
+    dw0, dw1, dw2 = O.fast_weight_grads(w0, w1, w2, k, v, lr0, lr1, lr2, F64)
+
+    def orth(G):
+        U, s, Vh = torch.linalg.svd(G, full_matrices=False)
+        return (U * _poly(s / (s.norm() + 1e-7), O.NS5_COEFFS)) @ Vh
+    for i in range(w0.shape[0]):
+        got = torch.cat([n0[i] - w0[i], n2[i] - w2[i]], dim=0)
+        assert torch.allclose(got, orth(torch.cat([dw0[i], dw2[i]], dim=0)), atol=1e-9)
+        assert torch.allclose(n1[i] - w1[i], orth(dw1[i]), atol=1e-9)
+        separate = torch.cat([orth(dw0[i]), orth(dw2[i])], dim=0)
+        assert not torch.allclose(got, separate, atol=1e-3)
+
+
+def test_fused_variant_renorm_has_eps_inside_the_sqrt():
+    """Row norms after y = x / sqrt(|x|^2 + eps) * n: |y| = n |x| / sqrt(|x|^2 + 1e-5); with |x|^2 ~ eps the two
+    conventions differ by tens of percent, so the check separates them."""
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(2, 4, 9, generator=g, dtype=torch.float64) * 1e-3
+    n = torch.rand(2, 4, 1, generator=g, dtype=torch.float64) + 0.5
+    y = O.renorm(x, n, F64, eps_in_sqrt=True)
+    xn = x.norm(dim=2, keepdim=True)
+    assert torch.allclose(y.norm(dim=2, keepdim=True), n * xn / torch.sqrt(xn ** 2 + 1e-5), rtol=1e-6)   # fp32 statistics
+    assert torch.allclose(y / y.norm(dim=2, keepdim=True), x / xn, atol=1e-6)                            # direction kept
+    y_out = O.renorm(x, n, F64)
+    assert torch.allclose(y_out.norm(dim=2, keepdim=True), n * xn / (xn + 1e-5), rtol=1e-10)
+    assert (y.norm(dim=2) / y_out.norm(dim=2) - 1).abs().min() > 0.05
+
+
+def test_fused_variant_entry_points_share_schedule_and_differ_only_in_the_two_switches():
+    w0, w1, w2, q, k, v, lr0, lr1, lr2 = rand_problem(b=2, L=50, d=6, dh=5)
+    mom = torch.sigmoid(torch.randn(2, 50, 1, dtype=torch.float64))
+    # without Muon the post-norm variants differ only through eps placement: at these row norms (~1) by ~1e-5
+    a = O.postnorm_block_causal_lact_swiglu_fused_kernel_triton(w0, w1, w2, q, k, v, lr0, lr1, lr2, 16, False, mom, num=F64)
+    b_ = O.block_causal_lact_swiglu(w0, w1, w2, q, k, v, lr0, lr1, lr2, 16, False, mom, num=F64)
+    assert a.shape == b_.shape and 0 < O.rel_l2(a, b_) < 1e-4
+    # pre-norm without Muon: identical (eps stays outside, :322-327)
+    a = O.prenorm_block_causal_lact_swiglu_fused_kernel_triton(w0, w1, w2, q, k, v, lr0, lr1, lr2, 16, False, mom, num=F64)
+    b_ = O.prenorm_block_causal_lact_swiglu(w0, w1, w2, q, k, v, lr0, lr1, lr2, 16, False, mom, num=F64)
+    assert torch.equal(a, b_)
+    # with Muon the stacking changes the result visibly, the first chunk (no update yet) not at all
+    a = O.prenorm_block_causal_lact_swiglu_fused_kernel_triton(w0, w1, w2, q, k, v, lr0, lr1, lr2, 16, True, mom, num=F64)
+    b_ = O.prenorm_block_causal_lact_swiglu(w0, w1, w2, q, k, v, lr0, lr1, lr2, 16, True, mom, num=F64)
+    assert torch.equal(a[:, :16], b_[:, :16]) and O.rel_l2(a[:, 16:], b_[:, 16:]) > 1e-3
