@@ -106,6 +106,39 @@ size_t lact_newton_schulz_workspace_bytes(int32_t n, int32_t rows, int32_t cols,
 int lact_newton_schulz(int32_t n, int32_t rows, int32_t cols, const float* g, float* out, int32_t steps,
                        const float* coeffs, int32_t ns_mode, void* workspace, void* stream);
 
+/* ---- Layer pre- and post-processing (the tensor code of the layer classes around the operation, one pass each;
+ * in the reference a chain of PyTorch ops in the layers' forward, with autograd for the backward).
+ * act_dtype as above; head dim a multiple of 4, at most 1024.  All buffers contiguous.
+ *
+ * pre: qkv [B, L, 3, H, hd] (output of the layer's to_qkv projection) -> q, k, v [(B H), L, hd]:
+ *      silu, L2 norm of q and k per head (x / (|x| + 1e-5)) when l2norm, head layout
+ *      (bidirectional_lact_layer.py:231-244; causal_lact_with_sliding_window_attn.py:313-322). */
+int lact_layer_pre_forward(int32_t act_dtype, int32_t B, int32_t L, int32_t H, int32_t hd, int32_t l2norm,
+                           const void* qkv, void* q, void* k, void* v, void* stream);
+int lact_layer_pre_backward(int32_t act_dtype, int32_t B, int32_t L, int32_t H, int32_t hd, int32_t l2norm,
+                            const void* qkv, const void* dq, const void* dk, const void* dv, void* dqkv,
+                            void* stream);
+/* lr: lr_raw [B, L, H, 3] fp32 (output of lr_proj) -> lr0, lr1, lr2 [(B H), L] = softplus(raw + base_lr_inv);
+ *     momentum_raw [B, L, H] fp32 (nullable; output of the linear map of momentum_proj) -> sigmoid, [(B H), L]
+ *     (bidirectional_lact_layer.py:248-256; causal_lact_with_sliding_window_attn.py:326-345). */
+int lact_layer_lr_forward(int32_t B, int32_t L, int32_t H, float base_lr_inv, const float* lr_raw, float* lr0,
+                          float* lr1, float* lr2, const float* momentum_raw, float* momentum, void* stream);
+int lact_layer_lr_backward(int32_t B, int32_t L, int32_t H, float base_lr_inv, const float* lr_raw,
+                           const float* dlr0, const float* dlr1, const float* dlr2, float* dlr_raw,
+                           const float* momentum_raw, const float* dmomentum, float* dmomentum_raw, void* stream);
+/* post: o [(B H), L, hd] (output of the operation) -> y [B, L, H*hd]: RMSNorm over the head dim with weight
+ *      norm_weight [hd] fp32 (nullable = ones) when use_norm, times silu(gate_raw [B, L, H]) when gate_raw is
+ *      given, head layout (bidirectional_lact_layer.py:268-270; causal_lact_with_sliding_window_attn.py:351-357).
+ *      The backward writes lact_layer_post_dw_rows(B, L, H) partial rows of the weight gradient into
+ *      dw_part [rows][hd] fp32 (the caller sums them), d_o and dgate_raw. */
+int lact_layer_post_forward(int32_t act_dtype, int32_t B, int32_t L, int32_t H, int32_t hd, int32_t use_norm,
+                            float eps, const void* o, const float* norm_weight, const void* gate_raw, void* y,
+                            void* stream);
+int32_t lact_layer_post_dw_rows(int32_t B, int32_t L, int32_t H);
+int lact_layer_post_backward(int32_t act_dtype, int32_t B, int32_t L, int32_t H, int32_t hd, int32_t use_norm,
+                             float eps, const void* o, const float* norm_weight, const void* gate_raw,
+                             const void* dy, void* d_o, void* dgate_raw, float* dw_part, void* stream);
+
 /* Execution options (process-wide; no counterpart in the reference, where PyTorch enqueues the whole layer on one
  * stream as separate kernels).  Both are on by default and change no result bit.
  *   LACT_OPT_STREAM_OVERLAP: the apply steps of a program do not depend on the update chain that runs beside
@@ -113,7 +146,7 @@ int lact_newton_schulz(int32_t n, int32_t rows, int32_t cols, const float* g, fl
  *     per device, created on first use) that is forked from and joined back into the caller's stream with
  *     events, so the call as a whole stays asynchronous and ordered on the caller's stream.
  *   LACT_OPT_FUSED_NEWTON_SCHULZ: all Newton-Schulz iterations of an update (and of its backward) run as one
- *     kernel whose blocks meet at per-matrix barriers (bf16, rows and columns multiples of 192, at most 8
+ *     kernel whose blocks meet at per-matrix barriers (bf16, rows and columns multiples of 192 or of 128, at most 8
  *     iterations); otherwise three GEMM launches per iteration.
  * Returns the previous value (0 / 1), or -1 for an unknown option. */
 enum { LACT_OPT_STREAM_OVERLAP = 0, LACT_OPT_FUSED_NEWTON_SCHULZ = 1 };

@@ -5,6 +5,8 @@ The package mirrors the reference's call signatures for this one path:
   lact_amd.minimal        <- minimal_implementations/*.py (operations)
   lact_amd.nvs            <- lact_nvs/lact_ttt.py (operation)
   lact_amd.ar_video       <- lact_ar_video/minVid/models/blocks/ar_lact_swa_repeat{,_sp}.py (operations)
+  lact_amd.layers         <- minimal_implementations/bidirectional_lact_layer.py, causal_lact_with_sliding_window_attn.py
+                             (the two layer classes around the operation)
 All arithmetic runs in lib/liblact_hip.so (built from csrc/ with hipcc for gfx950)."""
 from .ops import NS5_COEFFS, NS_CLASSIC, Program, block_causal_steps, run_program  # noqa: F401
 from .ttt_operation import (block_causal_lact_swiglu, l2_norm, prenorm_block_causal_lact_swiglu,  # noqa: F401
@@ -13,3 +15,4 @@ from .ttt_operation import (block_causal_lact_swiglu, l2_norm, prenorm_block_cau
                             silu_backprop, zeropower_via_newtonschulz5)
 from .minimal import bidirectional_lact_swiglu, inv_softplus  # noqa: F401
 from .nvs import TTTOperator, fast_weight_swish_glu_weight_norm_mini_batch_apply  # noqa: F401
+from .layers import BidirectionalLaCTSwiGLU, CausalLaCTSwiGLUWithSlidingWindowAttn, sliding_window_attention  # noqa: F401

@@ -36,7 +36,8 @@ class Desc(Structure):
 OPT_STREAM_OVERLAP, OPT_FUSED_NEWTON_SCHULZ = 0, 1
 EXPORTS = ("lact_last_error", "lact_version", "lact_query_sizes", "lact_forward", "lact_backward",
            "lact_newton_schulz_workspace_bytes", "lact_newton_schulz", "lact_set_option", "lact_profile_enable",
-           "lact_profile_report")
+           "lact_profile_report", "lact_layer_pre_forward", "lact_layer_pre_backward", "lact_layer_lr_forward",
+           "lact_layer_lr_backward", "lact_layer_post_forward", "lact_layer_post_dw_rows", "lact_layer_post_backward")
 
 _lib = None
 
@@ -65,6 +66,17 @@ def lib():
     L.lact_newton_schulz.restype = c_int32
     L.lact_set_option.argtypes = [c_int32, c_int32]
     L.lact_set_option.restype = c_int32
+    i32, f32 = c_int32, c_float
+    L.lact_layer_pre_forward.argtypes = [i32] * 6 + [vp] * 5
+    L.lact_layer_pre_backward.argtypes = [i32] * 6 + [vp] * 6
+    L.lact_layer_lr_forward.argtypes = [i32] * 3 + [f32] + [vp] * 7
+    L.lact_layer_lr_backward.argtypes = [i32] * 3 + [f32] + [vp] * 9
+    L.lact_layer_post_forward.argtypes = [i32] * 6 + [f32] + [vp] * 5
+    L.lact_layer_post_dw_rows.argtypes = [i32] * 3
+    L.lact_layer_post_backward.argtypes = [i32] * 6 + [f32] + [vp] * 8
+    for fn in ("lact_layer_pre_forward", "lact_layer_pre_backward", "lact_layer_lr_forward", "lact_layer_lr_backward",
+               "lact_layer_post_forward", "lact_layer_post_dw_rows", "lact_layer_post_backward"):
+        getattr(L, fn).restype = c_int32
     L.lact_profile_enable.argtypes = [c_int32]
     L.lact_profile_enable.restype = c_int32
     L.lact_profile_report.argtypes = [c_char_p, c_size_t]

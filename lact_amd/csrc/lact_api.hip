@@ -17,6 +17,7 @@
 #include "ns_fused.h"
 #include "gemm_kernels.h"
 #include "state_kernels.h"
+#include "layer_kernels.h"
 
 using namespace lact;
 
@@ -1212,6 +1213,120 @@ int lact_set_option(int32_t option, int32_t value) {
   const int was = *flag ? 1 : 0;
   *flag = value != 0;
   return was;
+}
+
+// ---- layer pre- and post-processing -----------------------------------------------------------------
+namespace {
+int layer_geom(int32_t B, int32_t L, int32_t H, int32_t hd, LayerGeom* g) {
+  if (B <= 0 || L <= 0 || H <= 0 || hd <= 0) return fail("layer: B, L, H, hd must be positive");
+  if (hd % 4 || hd > 256 * LAYER_VEC_MAX) return fail("layer: head dim must be a multiple of 4 and at most 1024");
+  g->B = B; g->L = L; g->H = H; g->hd = hd;
+  return 0;
+}
+unsigned layer_row_blocks(const LayerGeom& g) { return (unsigned)(((long long)g.B * g.L * g.H + 3) / 4); }
+unsigned layer_post_bwd_blocks(const LayerGeom& g) { return std::min(layer_row_blocks(g), 2048u); }
+}  // namespace
+
+int lact_layer_pre_forward(int32_t act_dtype, int32_t B, int32_t L, int32_t H, int32_t hd, int32_t l2norm, const void* qkv,
+                           void* q, void* k, void* v, void* stream) {
+  LayerPreParams p;
+  memset(&p, 0, sizeof(p));
+  if (layer_geom(B, L, H, hd, &p.g)) return -1;
+  if (check_ptrs({qkv, q, k, v}, "layer pre tensors")) return -1;
+  p.l2norm = l2norm; p.qkv = qkv; p.out[0] = q; p.out[1] = k; p.out[2] = v;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (act_dtype == LACT_BF16) LACT_LAUNCH("k_layer_pre", "layer_pre", 0.0, (k_layer_pre<uint16_t, false>), dim3(layer_row_blocks(p.g)), dim3(256), s, p);
+  else if (act_dtype == LACT_F32) LACT_LAUNCH("k_layer_pre", "layer_pre", 0.0, (k_layer_pre<float, false>), dim3(layer_row_blocks(p.g)), dim3(256), s, p);
+  else return fail("act_dtype must be LACT_BF16 or LACT_F32");
+  LACT_CHECK_LAUNCH();
+  return 0;
+}
+
+int lact_layer_pre_backward(int32_t act_dtype, int32_t B, int32_t L, int32_t H, int32_t hd, int32_t l2norm, const void* qkv,
+                            const void* dq, const void* dk, const void* dv, void* dqkv, void* stream) {
+  LayerPreParams p;
+  memset(&p, 0, sizeof(p));
+  if (layer_geom(B, L, H, hd, &p.g)) return -1;
+  if (check_ptrs({qkv, dq, dk, dv, dqkv}, "layer pre backward tensors")) return -1;
+  p.l2norm = l2norm; p.qkv = qkv; p.dout[0] = dq; p.dout[1] = dk; p.dout[2] = dv; p.dqkv = dqkv;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (act_dtype == LACT_BF16) LACT_LAUNCH("k_layer_pre_bwd", "layer_pre_bwd", 0.0, (k_layer_pre<uint16_t, true>), dim3(layer_row_blocks(p.g)), dim3(256), s, p);
+  else if (act_dtype == LACT_F32) LACT_LAUNCH("k_layer_pre_bwd", "layer_pre_bwd", 0.0, (k_layer_pre<float, true>), dim3(layer_row_blocks(p.g)), dim3(256), s, p);
+  else return fail("act_dtype must be LACT_BF16 or LACT_F32");
+  LACT_CHECK_LAUNCH();
+  return 0;
+}
+
+int lact_layer_lr_forward(int32_t B, int32_t L, int32_t H, float base_lr_inv, const float* lr_raw, float* lr0, float* lr1,
+                          float* lr2, const float* momentum_raw, float* momentum, void* stream) {
+  LayerLrParams p;
+  memset(&p, 0, sizeof(p));
+  if (layer_geom(B, L, H, 4, &p.g)) return -1;
+  if (check_ptrs({lr_raw, lr0, lr1, lr2}, "layer lr tensors")) return -1;
+  if (momentum_raw && !momentum) return fail("momentum_raw given without momentum output");
+  p.base_lr_inv = base_lr_inv; p.lr_raw = lr_raw; p.lr[0] = lr0; p.lr[1] = lr1; p.lr[2] = lr2;
+  p.mom_raw = momentum_raw; p.mom = momentum;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const long long n = (long long)B * L * H;
+  LACT_LAUNCH("k_layer_lr", "layer_lr", 0.0, (k_layer_lr<false>), dim3((unsigned)((n + 255) / 256)), dim3(256), s, p);
+  LACT_CHECK_LAUNCH();
+  return 0;
+}
+
+int lact_layer_lr_backward(int32_t B, int32_t L, int32_t H, float base_lr_inv, const float* lr_raw, const float* dlr0,
+                           const float* dlr1, const float* dlr2, float* dlr_raw, const float* momentum_raw,
+                           const float* dmomentum, float* dmomentum_raw, void* stream) {
+  LayerLrParams p;
+  memset(&p, 0, sizeof(p));
+  if (layer_geom(B, L, H, 4, &p.g)) return -1;
+  if (check_ptrs({lr_raw, dlr_raw}, "layer lr backward tensors")) return -1;
+  if (momentum_raw && !dmomentum_raw) return fail("momentum_raw given without dmomentum_raw output");
+  p.base_lr_inv = base_lr_inv; p.lr_raw = lr_raw; p.dlr[0] = dlr0; p.dlr[1] = dlr1; p.dlr[2] = dlr2; p.dlr_raw = dlr_raw;
+  p.mom_raw = momentum_raw; p.dmom = dmomentum; p.dmom_raw = dmomentum_raw;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const long long n = (long long)B * L * H;
+  LACT_LAUNCH("k_layer_lr_bwd", "layer_lr_bwd", 0.0, (k_layer_lr<true>), dim3((unsigned)((n + 255) / 256)), dim3(256), s, p);
+  LACT_CHECK_LAUNCH();
+  return 0;
+}
+
+int lact_layer_post_forward(int32_t act_dtype, int32_t B, int32_t L, int32_t H, int32_t hd, int32_t use_norm, float eps,
+                            const void* o, const float* norm_weight, const void* gate_raw, void* y, void* stream) {
+  LayerPostParams p;
+  memset(&p, 0, sizeof(p));
+  if (layer_geom(B, L, H, hd, &p.g)) return -1;
+  if (check_ptrs({o, y}, "layer post tensors")) return -1;
+  p.eps = eps; p.use_norm = use_norm; p.o = o; p.w = norm_weight; p.gate_raw = gate_raw; p.y = y;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (act_dtype == LACT_BF16) LACT_LAUNCH("k_layer_post", "layer_post", 0.0, (k_layer_post<uint16_t, false>), dim3(layer_row_blocks(p.g)), dim3(256), s, p);
+  else if (act_dtype == LACT_F32) LACT_LAUNCH("k_layer_post", "layer_post", 0.0, (k_layer_post<float, false>), dim3(layer_row_blocks(p.g)), dim3(256), s, p);
+  else return fail("act_dtype must be LACT_BF16 or LACT_F32");
+  LACT_CHECK_LAUNCH();
+  return 0;
+}
+
+int32_t lact_layer_post_dw_rows(int32_t B, int32_t L, int32_t H) {
+  LayerGeom g;
+  if (layer_geom(B, L, H, 4, &g)) return -1;
+  return (int32_t)layer_post_bwd_blocks(g) * 4;
+}
+
+int lact_layer_post_backward(int32_t act_dtype, int32_t B, int32_t L, int32_t H, int32_t hd, int32_t use_norm, float eps,
+                             const void* o, const float* norm_weight, const void* gate_raw, const void* dy, void* d_o,
+                             void* dgate_raw, float* dw_part, void* stream) {
+  LayerPostParams p;
+  memset(&p, 0, sizeof(p));
+  if (layer_geom(B, L, H, hd, &p.g)) return -1;
+  if (check_ptrs({o, dy, d_o}, "layer post backward tensors")) return -1;
+  if (gate_raw && !dgate_raw) return fail("gate_raw given without dgate_raw output");
+  p.eps = eps; p.use_norm = use_norm; p.o = o; p.w = norm_weight; p.gate_raw = gate_raw;
+  p.dy = dy; p.d_o = d_o; p.dgate_raw = dgate_raw; p.dw_part = use_norm ? dw_part : nullptr;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (act_dtype == LACT_BF16) LACT_LAUNCH("k_layer_post_bwd", "layer_post_bwd", 0.0, (k_layer_post<uint16_t, true>), dim3(layer_post_bwd_blocks(p.g)), dim3(256), s, p);
+  else if (act_dtype == LACT_F32) LACT_LAUNCH("k_layer_post_bwd", "layer_post_bwd", 0.0, (k_layer_post<float, true>), dim3(layer_post_bwd_blocks(p.g)), dim3(256), s, p);
+  else return fail("act_dtype must be LACT_BF16 or LACT_F32");
+  LACT_CHECK_LAUNCH();
+  return 0;
 }
 
 int lact_profile_enable(int on) {
