@@ -118,12 +118,13 @@ int lact_layer_pre_forward(int32_t act_dtype, int32_t B, int32_t L, int32_t H, i
 int lact_layer_pre_backward(int32_t act_dtype, int32_t B, int32_t L, int32_t H, int32_t hd, int32_t l2norm,
                             const void* qkv, const void* dq, const void* dk, const void* dv, void* dqkv,
                             void* stream);
-/* lr: lr_raw [B, L, H, 3] fp32 (output of lr_proj) -> lr0, lr1, lr2 [(B H), L] = softplus(raw + base_lr_inv);
+/* lr: lr_raw fp32 (output of lr_proj) -> lr0, lr1, lr2 [(B H), L] = softplus(raw + base_lr_inv); lr_raw is
+ *     [B, L, H, 3] ('b l (h lrs d)') when rates_major == 0 and [B, L, 3, H] ('b l (lrs h d)', lact_ttt.py:213-216) else;
  *     momentum_raw [B, L, H] fp32 (nullable; output of the linear map of momentum_proj) -> sigmoid, [(B H), L]
  *     (bidirectional_lact_layer.py:248-256; causal_lact_with_sliding_window_attn.py:326-345). */
-int lact_layer_lr_forward(int32_t B, int32_t L, int32_t H, float base_lr_inv, const float* lr_raw, float* lr0,
+int lact_layer_lr_forward(int32_t B, int32_t L, int32_t H, int32_t rates_major, float base_lr_inv, const float* lr_raw, float* lr0,
                           float* lr1, float* lr2, const float* momentum_raw, float* momentum, void* stream);
-int lact_layer_lr_backward(int32_t B, int32_t L, int32_t H, float base_lr_inv, const float* lr_raw,
+int lact_layer_lr_backward(int32_t B, int32_t L, int32_t H, int32_t rates_major, float base_lr_inv, const float* lr_raw,
                            const float* dlr0, const float* dlr1, const float* dlr2, float* dlr_raw,
                            const float* momentum_raw, const float* dmomentum, float* dmomentum_raw, void* stream);
 /* post: o [(B H), L, hd] (output of the operation) -> y [B, L, H*hd]: RMSNorm over the head dim with weight

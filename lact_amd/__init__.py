@@ -15,4 +15,5 @@ from .ttt_operation import (block_causal_lact_swiglu, l2_norm, prenorm_block_cau
                             silu_backprop, zeropower_via_newtonschulz5)
 from .minimal import bidirectional_lact_swiglu, inv_softplus  # noqa: F401
 from .nvs import TTTOperator, fast_weight_swish_glu_weight_norm_mini_batch_apply  # noqa: F401
-from .layers import BidirectionalLaCTSwiGLU, CausalLaCTSwiGLUWithSlidingWindowAttn, sliding_window_attention  # noqa: F401
+from .layers import (BidirectionalLaCTSwiGLU, CausalLaCTSwiGLUWithSlidingWindowAttn, FastWeightGluMLPMultihead,  # noqa: F401
+                     sliding_window_attention)

@@ -69,8 +69,8 @@ def lib():
     i32, f32 = c_int32, c_float
     L.lact_layer_pre_forward.argtypes = [i32] * 6 + [vp] * 5
     L.lact_layer_pre_backward.argtypes = [i32] * 6 + [vp] * 6
-    L.lact_layer_lr_forward.argtypes = [i32] * 3 + [f32] + [vp] * 7
-    L.lact_layer_lr_backward.argtypes = [i32] * 3 + [f32] + [vp] * 9
+    L.lact_layer_lr_forward.argtypes = [i32] * 4 + [f32] + [vp] * 7
+    L.lact_layer_lr_backward.argtypes = [i32] * 4 + [f32] + [vp] * 9
     L.lact_layer_post_forward.argtypes = [i32] * 6 + [f32] + [vp] * 5
     L.lact_layer_post_dw_rows.argtypes = [i32] * 3
     L.lact_layer_post_backward.argtypes = [i32] * 6 + [f32] + [vp] * 8

@@ -1257,13 +1257,14 @@ int lact_layer_pre_backward(int32_t act_dtype, int32_t B, int32_t L, int32_t H, 
   return 0;
 }
 
-int lact_layer_lr_forward(int32_t B, int32_t L, int32_t H, float base_lr_inv, const float* lr_raw, float* lr0, float* lr1,
+int lact_layer_lr_forward(int32_t B, int32_t L, int32_t H, int32_t rates_major, float base_lr_inv, const float* lr_raw, float* lr0, float* lr1,
                           float* lr2, const float* momentum_raw, float* momentum, void* stream) {
   LayerLrParams p;
   memset(&p, 0, sizeof(p));
   if (layer_geom(B, L, H, 4, &p.g)) return -1;
   if (check_ptrs({lr_raw, lr0, lr1, lr2}, "layer lr tensors")) return -1;
   if (momentum_raw && !momentum) return fail("momentum_raw given without momentum output");
+  p.rates_major = rates_major != 0;
   p.base_lr_inv = base_lr_inv; p.lr_raw = lr_raw; p.lr[0] = lr0; p.lr[1] = lr1; p.lr[2] = lr2;
   p.mom_raw = momentum_raw; p.mom = momentum;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
@@ -1273,7 +1274,7 @@ int lact_layer_lr_forward(int32_t B, int32_t L, int32_t H, float base_lr_inv, co
   return 0;
 }
 
-int lact_layer_lr_backward(int32_t B, int32_t L, int32_t H, float base_lr_inv, const float* lr_raw, const float* dlr0,
+int lact_layer_lr_backward(int32_t B, int32_t L, int32_t H, int32_t rates_major, float base_lr_inv, const float* lr_raw, const float* dlr0,
                            const float* dlr1, const float* dlr2, float* dlr_raw, const float* momentum_raw,
                            const float* dmomentum, float* dmomentum_raw, void* stream) {
   LayerLrParams p;
@@ -1281,6 +1282,7 @@ int lact_layer_lr_backward(int32_t B, int32_t L, int32_t H, float base_lr_inv, c
   if (layer_geom(B, L, H, 4, &p.g)) return -1;
   if (check_ptrs({lr_raw, dlr_raw}, "layer lr backward tensors")) return -1;
   if (momentum_raw && !dmomentum_raw) return fail("momentum_raw given without dmomentum_raw output");
+  p.rates_major = rates_major != 0;
   p.base_lr_inv = base_lr_inv; p.lr_raw = lr_raw; p.dlr[0] = dlr0; p.dlr[1] = dlr1; p.dlr[2] = dlr2; p.dlr_raw = dlr_raw;
   p.mom_raw = momentum_raw; p.dmom = dmomentum; p.dmom_raw = dmomentum_raw;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);

@@ -118,7 +118,8 @@ __global__ __launch_bounds__(256) void k_layer_pre(const LayerPreParams p) {
 struct LayerLrParams {
   LayerGeom g;
   float base_lr_inv;
-  const float* lr_raw;        // [B, L, H, 3]
+  const float* lr_raw;        // [B, L, H, 3], or [B, L, 3, H] when rates_major
+  int rates_major;
   float* lr[3];               // [(B H), L]
   const float* mom_raw;       // [B, L, H] or null
   float* mom;                 // [(B H), L]
@@ -137,9 +138,10 @@ __global__ void k_layer_lr(const LayerLrParams p) {
   const size_t o = (size_t)(b * p.g.H + h) * p.g.L + l;
 #pragma unroll
   for (int s = 0; s < 3; ++s) {
-    const float x = p.lr_raw[i * 3 + s] + p.base_lr_inv;
+    const long long ri = p.rates_major ? (bl * 3 + s) * p.g.H + h : i * 3 + s;
+    const float x = p.lr_raw[ri] + p.base_lr_inv;
     if (!BWD) p.lr[s][o] = x > 20.f ? x : log1pf(__expf(x));          // softplus (threshold as in torch)
-    else p.dlr_raw[i * 3 + s] = p.dlr[s] ? p.dlr[s][o] * (x > 20.f ? 1.f : sigmoidf_(x)) : 0.f;
+    else p.dlr_raw[ri] = p.dlr[s] ? p.dlr[s][o] * (x > 20.f ? 1.f : sigmoidf_(x)) : 0.f;
   }
   if (p.mom_raw) {
     const float s = sigmoidf_(p.mom_raw[i]);

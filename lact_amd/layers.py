@@ -3,6 +3,7 @@ arguments and parameter names (a state_dict moves over unchanged):
 
   BidirectionalLaCTSwiGLU                minimal_implementations/bidirectional_lact_layer.py:171-270
   CausalLaCTSwiGLUWithSlidingWindowAttn  minimal_implementations/causal_lact_with_sliding_window_attn.py:222-391
+  FastWeightGluMLPMultihead              lact_nvs/lact_ttt.py:150-258
 
 The projections are torch.nn.Linear (hipBLASLt).  Everything between them runs in liblact_hip.so: one kernel turns
 the to_qkv output into the operation's q, k, v (silu, per-head L2 norm, head layout), one makes the learning rates
@@ -24,6 +25,7 @@ import torch.nn.functional as F
 from . import _lib
 from ._lib import LACT_BF16, LACT_F32
 from .minimal import bidirectional_lact_swiglu, block_causal_lact_swiglu, inv_softplus
+from .nvs import fast_weight_swish_glu_weight_norm_mini_batch_apply
 
 
 def _ptr(t: Optional[torch.Tensor]):
@@ -73,22 +75,22 @@ class _PreFn(torch.autograd.Function):
 
 
 class _LrFn(torch.autograd.Function):
-    """lr_raw [B, L, 3*H] (head-major, three rates per head), momentum_raw [B, L, H] or None
-    -> lr0, lr1, lr2, momentum [(B H), L, 1] fp32."""
+    """lr_raw [B, L, 3*H] (head-major with three rates per head, or rate-major when rates_major), momentum_raw
+    [B, L, H] or None -> lr0, lr1, lr2, momentum [(B H), L, 1] fp32."""
 
     @staticmethod
-    def forward(ctx, lr_raw, mom_raw, H, base_lr_inv):
+    def forward(ctx, lr_raw, mom_raw, H, base_lr_inv, rates_major=False):
         lr_raw = lr_raw.float().contiguous()
         mom_c = None if mom_raw is None else mom_raw.float().contiguous()
         B, L, _ = lr_raw.shape
         outs = [torch.empty((B * H, L, 1), dtype=torch.float32, device=lr_raw.device) for _ in range(3)]
         mom = torch.empty((B * H, L, 1), dtype=torch.float32, device=lr_raw.device) if mom_c is not None else None
         with torch.cuda.device(lr_raw.device):
-            _lib.check(_lib.lib().lact_layer_lr_forward(B, L, H, float(base_lr_inv), _ptr(lr_raw), _ptr(outs[0]),
+            _lib.check(_lib.lib().lact_layer_lr_forward(B, L, H, int(rates_major), float(base_lr_inv), _ptr(lr_raw), _ptr(outs[0]),
                                                         _ptr(outs[1]), _ptr(outs[2]), _ptr(mom_c), _ptr(mom),
                                                         _stream(lr_raw)))
         ctx.save_for_backward(lr_raw, mom_c)
-        ctx.dims = (B, L, H, float(base_lr_inv))
+        ctx.dims = (B, L, H, float(base_lr_inv), int(rates_major))
         ctx.mom_dtype = None if mom_raw is None else mom_raw.dtype
         if mom is None:
             return outs[0], outs[1], outs[2]
@@ -97,16 +99,16 @@ class _LrFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, d0, d1, d2, dm=None):
         lr_raw, mom_c = ctx.saved_tensors
-        B, L, H, base = ctx.dims
+        B, L, H, base, rates_major = ctx.dims
         c = lambda g: None if g is None else g.float().contiguous()
         d0, d1, d2, dm = c(d0), c(d1), c(d2), c(dm)
         dlr_raw = torch.empty_like(lr_raw)
         dmom_raw = torch.empty_like(mom_c) if mom_c is not None else None
         with torch.cuda.device(lr_raw.device):
-            _lib.check(_lib.lib().lact_layer_lr_backward(B, L, H, base, _ptr(lr_raw), _ptr(d0), _ptr(d1), _ptr(d2),
+            _lib.check(_lib.lib().lact_layer_lr_backward(B, L, H, rates_major, base, _ptr(lr_raw), _ptr(d0), _ptr(d1), _ptr(d2),
                                                          _ptr(dlr_raw), _ptr(mom_c), _ptr(dm), _ptr(dmom_raw),
                                                          _stream(lr_raw)))
-        return dlr_raw, (None if dmom_raw is None else dmom_raw.to(ctx.mom_dtype)), None, None
+        return dlr_raw, (None if dmom_raw is None else dmom_raw.to(ctx.mom_dtype)), None, None, None
 
 
 class _PostFn(torch.autograd.Function):
@@ -267,3 +269,47 @@ class CausalLaCTSwiGLUWithSlidingWindowAttn(nn.Module):
         sh = lambda t: t.reshape(B, L, self.num_attn_heads, self.attn_head_dim)
         attn = sliding_window_attention(sh(aq), sh(ak), sh(av), self.window_size).reshape(B, L, -1)
         return self.o_proj(attn + ttt)
+
+
+class FastWeightGluMLPMultihead(nn.Module):
+    """lact_nvs/lact_ttt.py:150-258: the layer of the novel-view-synthesis model.  Fast weights in the transposed
+    layout (w0, w2: [nh, d, dh]; w1: [nh, dh, d]); `info["ttt_op_order"]` is the list of TTTOperator steps and
+    `info["w0"/"w1"/"w2"]`, when present, are the fast weights a previous call returned (state carried from the
+    reconstruction pass into the rendering pass, lact_nvs/model.py:272-384)."""
+
+    def __init__(self, dim: int, head_dim: int, inter_multi: int = 1, bias: bool = False, base_lr: float = 0.01,
+                 muon_update_steps: int = 0):
+        super().__init__()
+        assert dim % head_dim == 0
+        self.dim, self.num_heads, self.muon_update_steps = dim, dim // head_dim, muon_update_steps
+        self.head_dim = head_dim
+        d_in = d_out = head_dim
+        d_h = int(head_dim * inter_multi)
+        gain = math.sqrt(2)
+        self.w0 = nn.Parameter(torch.randn(self.num_heads, d_in, d_h) * gain / math.sqrt(d_in))
+        self.w1 = nn.Parameter(torch.randn(self.num_heads, d_h, d_out) * gain / math.sqrt(d_h))
+        self.w2 = nn.Parameter(torch.randn(self.num_heads, d_in, d_h) * gain / math.sqrt(d_in))
+        self.to_qkv = nn.Linear(dim, 3 * dim, bias=bias)
+        self.c_proj = nn.Linear(dim, dim, bias=bias)
+        self.lr_dim = self.num_heads
+        self.lr_fc = nn.Linear(dim, self.lr_dim * 3)
+        self.base_lr_inv = inv_softplus(base_lr)
+        self.o_norm = nn.RMSNorm(head_dim, eps=1e-5, elementwise_affine=True)
+
+    def forward(self, x: torch.Tensor, info={}, *args):
+        """x: [b, l, d] -> ([b, l', d], {"w0", "w1", "w2"}) with l' the rows of the apply steps in program order."""
+        B = x.shape[0]
+        q, k, v = _PreFn.apply(self.to_qkv(x), self.num_heads, self.head_dim, True)          # :203-210
+        with torch.autocast(device_type="cuda", enabled=False):                              # :212-213
+            lr_raw = self.lr_fc(x.float())
+        lr0, lr1, lr2 = _LrFn.apply(lr_raw, None, self.num_heads, self.base_lr_inv, True)    # '(lrs h d)', :215-219
+        if "w0" in info:                                                                      # :221-229
+            assert "w1" in info and "w2" in info
+            w0, w1, w2 = info["w0"], info["w1"], info["w2"]
+        else:
+            w0, w1, w2 = _fast_weights(self, B)
+        o, w0, w1, w2 = fast_weight_swish_glu_weight_norm_mini_batch_apply(
+            w0, w1, w2, q, k, v, lr0, lr1, lr2, info["ttt_op_order"], muon_update_steps=self.muon_update_steps)
+        weight, use_norm, eps = _norm_args(self.o_norm)
+        y = _PostFn.apply(o, weight, None, B, self.num_heads, use_norm, eps)
+        return self.c_proj(y), {"w0": w0, "w1": w1, "w2": w2}

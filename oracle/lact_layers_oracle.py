@@ -3,6 +3,7 @@ nothing in the product imports this module; tests compare the HIP-backed layers 
 
   BidirectionalLaCTSwiGLU                minimal_implementations/bidirectional_lact_layer.py:171-270
   CausalLaCTSwiGLUWithSlidingWindowAttn  minimal_implementations/causal_lact_with_sliding_window_attn.py:222-391
+  FastWeightGluMLPMultihead              lact_nvs/lact_ttt.py:150-258
 
 Parameter names equal the reference's, so a state_dict moves between the three implementations.  The operation
 inside is the oracle's (oracle/lact_oracle.py).  The sliding-window attention of the causal layer, which the
@@ -12,6 +13,9 @@ softmax: query i sees keys j with i-(W-1) <= j <= i, scale 1/sqrt(attn_head_dim)
 Pinned by tests/golden/bidirectional_layer_cpu_fp32.npz (the reference's own bidirectional layer run on the CPU:
 output and every gradient); the causal layer shares all of that code path except momentum head, per-head gate,
 q/k rescale and the attention branch, which are pinned by closed-form checks in tests/test_oracle_layers.py.
+The novel-view-synthesis layer (rate-major learning-rate layout, transposed fast weights, weights carried through
+`info`) is pinned there too: against a per-head composition written with explicit loops, and by the identity
+"update in one call, apply in the next with the returned weights" == "update and apply in one call".
 """
 from __future__ import annotations
 
@@ -137,3 +141,42 @@ class CausalLaCTSwiGLUWithSlidingWindowAttn(nn.Module):
         sh = lambda t: t.reshape(B, L, self.num_attn_heads, self.attn_head_dim)
         attn = sliding_window_attention(sh(aq), sh(ak), sh(av), self.window_size).reshape(B, L, -1)   # :371-377
         return self.o_proj(attn + ttt)                                                 # :379-382
+
+
+class FastWeightGluMLPMultihead(nn.Module):
+    """lact_nvs/lact_ttt.py:150-258."""
+
+    def __init__(self, dim: int, head_dim: int, inter_multi: int = 1, bias: bool = False, base_lr: float = 0.01,
+                 muon_update_steps: int = 0, num: O.Numerics = O.Numerics()):
+        super().__init__()
+        self.dim, self.head_dim, self.num_heads = dim, head_dim, dim // head_dim
+        self.muon_update_steps = muon_update_steps
+        d_h = int(head_dim * inter_multi)
+        gain = math.sqrt(2)
+        self.w0 = nn.Parameter(torch.randn(self.num_heads, head_dim, d_h) * gain / math.sqrt(head_dim))   # :186-194
+        self.w1 = nn.Parameter(torch.randn(self.num_heads, d_h, head_dim) * gain / math.sqrt(d_h))
+        self.w2 = nn.Parameter(torch.randn(self.num_heads, head_dim, d_h) * gain / math.sqrt(head_dim))
+        self.to_qkv = nn.Linear(dim, 3 * dim, bias=bias)
+        self.c_proj = nn.Linear(dim, dim, bias=bias)
+        self.lr_fc = nn.Linear(dim, self.num_heads * 3)
+        self.base_lr_inv = O.inv_softplus(base_lr)
+        self.o_norm = nn.RMSNorm(head_dim, eps=1e-5, elementwise_affine=True)
+        self.num = num
+
+    def forward(self, x: torch.Tensor, info={}, *args):
+        B, L, _ = x.shape
+        H = self.num_heads
+        qkv = F.silu(self.to_qkv(x))                                                   # :203
+        q, k, v = _heads(qkv, 3, H, self.head_dim)                                     # :204-207
+        q, k = O.l2_norm(q, self.num), O.l2_norm(k, self.num)                          # :208-209
+        lr = F.softplus(self.lr_fc(x.to(torch.promote_types(x.dtype, torch.float32))) + self.base_lr_inv)   # :211-214
+        lr0, lr1, lr2 = _heads(lr, 3, H, 1)                                            # 'b l (lrs h d) -> lrs (b h) l d', :215-218
+        if "w0" in info:                                                               # :220-228
+            w0, w1, w2 = info["w0"], info["w1"], info["w2"]
+        else:
+            w0, w1, w2 = (w.repeat(B, 1, 1) for w in (self.w0, self.w1, self.w2))
+        o, w0, w1, w2 = O.fast_weight_swish_glu_weight_norm_mini_batch_apply(
+            w0, w1, w2, q, k, v, lr0, lr1, lr2, info["ttt_op_order"], muon_update_steps=self.muon_update_steps,
+            num=self.num)                                                              # :230-233
+        o = self.o_norm(o)                                                             # :235
+        return self.c_proj(_unheads(o, B, H)), {"w0": w0, "w1": w1, "w2": w2}          # :236-241

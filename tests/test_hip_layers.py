@@ -228,3 +228,43 @@ def test_causal_layer_bf16_autocast():
     say("  ", errs)
     assert res["y"].shape == ref["y"].shape
     assert max(errs.values()) < 3e-2
+
+
+@pytest.mark.parametrize("steps", [0, 3])
+def test_nvs_layer_against_oracle(steps):
+    """FastWeightGluMLPMultihead (lact_nvs/lact_ttt.py:150-258): a reconstruction call (update + apply) whose
+    returned fast weights feed a rendering call (apply only); output of both calls, the carried weights and every
+    gradient against the float64 oracle layer (Newton-Schulz in fp32 on the GPU: exact arithmetic on both sides)."""
+    say("nvs layer vs oracle, muon steps", steps)
+    torch.manual_seed(14)
+    kw = dict(dim=256, head_dim=64, inter_multi=2, bias=True, base_lr=0.01, muon_update_steps=steps)
+    ref_layer = LO.FastWeightGluMLPMultihead(num=EXACT, **kw)
+    with torch.no_grad():
+        ref_layer.o_norm.weight.uniform_(0.5, 1.5)
+    layer = HL.FastWeightGluMLPMultihead(**kw).to(DEV)
+    layer.load_state_dict(ref_layer.state_dict(), strict=True)
+    ref_layer = ref_layer.double()
+    x1, x2 = torch.randn(2, 160, 256), torch.randn(2, 72, 256)
+    go1, go2 = torch.randn(2, 100, 256), torch.randn(2, 72, 256)
+    order1 = [O.TTTOperator(0, 96, True, True), O.TTTOperator(96, 160, True, False), O.TTTOperator(60, 64, False, True)]
+    order2 = [O.TTTOperator(0, 72, False, True)]
+
+    def run(lay, a, b, ga, gb):
+        a = a.clone().requires_grad_(True)
+        b = b.clone().requires_grad_(True)
+        y1, st = lay(a, {"ttt_op_order": order1})
+        y2, st2 = lay(b, {"ttt_op_order": order2, **st})
+        (y1 * ga.to(y1.dtype)).sum().add((y2 * gb.to(y2.dtype)).sum()).backward()
+        res = {"y1": y1, "y2": y2, "w0": st["w0"], "w1": st["w1"], "w2": st["w2"], "dx1": a.grad, "dx2": b.grad}
+        res.update({"d." + n: p.grad for n, p in lay.named_parameters()})
+        res = {n: t.detach().float().cpu() for n, t in res.items()}
+        lay.zero_grad(set_to_none=True)
+        return res
+
+    ref = run(ref_layer, x1.double(), x2.double(), go1.double(), go2.double())
+    with ops.newton_schulz_mode(ops.NS_FP32):
+        res = run(layer, x1.to(DEV), x2.to(DEV), go1.to(DEV), go2.to(DEV))
+    errs = compare(res, ref)
+    say("  ", errs)
+    assert res["y1"].shape == (2, 100, 256) and res["y2"].shape == (2, 72, 256)
+    assert max(errs.values()) < 1e-3

@@ -123,3 +123,81 @@ def test_causal_layer_momentum_head_reaches_the_operation():
         y0 = layer(x)
         assert O.rel_l2(y1[:, 32:], y0[:, 32:]) > 1e-4         # momentum matters from the third chunk on
         assert torch.allclose(y1[:, :32], y0[:, :32], atol=1e-12)   # ... and not before (first update has no state)
+
+
+EXACT = O.Numerics(autocast=False, ns_dtype=None)
+
+
+def _nvs_layer(steps=0):
+    torch.manual_seed(5)
+    layer = LO.FastWeightGluMLPMultihead(dim=24, head_dim=8, inter_multi=2, bias=True, base_lr=0.02,
+                                         muon_update_steps=steps, num=EXACT).double()
+    with torch.no_grad():
+        layer.o_norm.weight.uniform_(0.5, 1.5)
+        layer.lr_fc.weight.mul_(3.0)       # rates that differ visibly between heads and between the three matrices
+    return layer
+
+
+def test_nvs_layer_against_per_head_composition():
+    """lact_nvs/lact_ttt.py:200-241 written out head by head with explicit loops and index arithmetic: one update on
+    rows [0, 12), then an apply on rows [4, 20) (Newton-Schulz with 0 iterations = Frobenius normalisation).  A wrong
+    rate layout ('(h lrs)' for '(lrs h)'), a wrong head split of qkv, transposed fast weights or a norm over the
+    wrong axis all fail it."""
+    layer = _nvs_layer()
+    B, L, D, H, hd = 2, 20, 24, 3, 8
+    x = torch.randn(B, L, D, dtype=torch.float64)
+    order = [O.TTTOperator(0, 12, True, False), O.TTTOperator(4, 20, False, True)]
+    with torch.no_grad():
+        y, st = layer(x, {"ttt_op_order": order})
+        qkv = F.silu(layer.to_qkv(x))
+        lr = F.softplus(layer.lr_fc(x) + layer.base_lr_inv)
+        heads = []
+        for b in range(B):
+            row = []
+            for h in range(H):
+                q = qkv[b, :, 0 * D + h * hd:0 * D + (h + 1) * hd]
+                k = qkv[b, :, 1 * D + h * hd:1 * D + (h + 1) * hd]
+                v = qkv[b, :, 2 * D + h * hd:2 * D + (h + 1) * hd]
+                q = q / (q.norm(dim=1, keepdim=True) + 1e-5)
+                k = k / (k.norm(dim=1, keepdim=True) + 1e-5)
+                l0, l1, l2 = (lr[b, :, s * H + h:s * H + h + 1] for s in range(3))
+                w0, w1, w2 = layer.w0[h], layer.w1[h], layer.w2[h]          # [d, dh], [dh, d], [d, dh]
+                n0, n1, n2 = (w.norm(dim=0, keepdim=True) for w in (w0, w1, w2))
+                ki, vi = k[:12], v[:12]
+                g, hb = ki @ w0, ki @ w2
+                hid = F.silu(g) * hb
+                dh_ = vi @ w1.T
+                dhb = dh_ * F.silu(g)
+                sg = torch.sigmoid(g)
+                dg = dh_ * hb * sg * (1 + g * (1 - sg))
+                fro = lambda m: m / (m.norm() + 1e-7)
+                w1n = w1 + fro((hid * l1[:12]).T @ vi)
+                w0n = w0 + fro((ki * l0[:12]).T @ dg)
+                w2n = w2 + fro((ki * l2[:12]).T @ dhb)
+                w0n = w0n / (w0n.norm(dim=0, keepdim=True) + 1e-5) * n0
+                w1n = w1n / (w1n.norm(dim=0, keepdim=True) + 1e-5) * n1
+                w2n = w2n / (w2n.norm(dim=0, keepdim=True) + 1e-5) * n2
+                assert torch.allclose(st["w0"][b * H + h], w0n, atol=1e-12)
+                assert torch.allclose(st["w1"][b * H + h], w1n, atol=1e-12)
+                o = (F.silu(q[4:20] @ w0n) * (q[4:20] @ w2n)) @ w1n
+                o = o * torch.rsqrt((o * o).mean(dim=1, keepdim=True) + 1e-5) * layer.o_norm.weight
+                row.append(o)
+            heads.append(torch.cat(row, dim=1))
+        ref = layer.c_proj(torch.stack(heads))
+    assert y.shape == (B, 16, D)
+    assert torch.allclose(y, ref, atol=1e-11)
+
+
+def test_nvs_layer_carries_weights_through_info():
+    """Update in one call and apply in the next with the returned weights == both in one call
+    (lact_nvs/model.py:272-384 runs reconstruction and rendering that way)."""
+    layer = _nvs_layer(steps=2)
+    x = torch.randn(2, 20, 24, dtype=torch.float64)
+    with torch.no_grad():
+        y_both, st_both = layer(x, {"ttt_op_order": [O.TTTOperator(0, 12, True, False), O.TTTOperator(0, 20, False, True)]})
+        _y, st = layer(x, {"ttt_op_order": [O.TTTOperator(0, 12, True, True)]})
+        y2, st2 = layer(x, {"ttt_op_order": [O.TTTOperator(0, 20, False, True)], **st})
+    assert torch.allclose(y2, y_both, atol=1e-12)
+    for n in ("w0", "w1", "w2"):
+        assert torch.equal(st2[n], st[n]) and torch.allclose(st[n], st_both[n], atol=1e-12)
+    assert not torch.allclose(st["w0"], layer.w0.repeat(2, 1, 1), atol=1e-3)
