@@ -437,10 +437,12 @@ struct Runner {
     return false;
   }
   unsigned* ns_error_word() const { return scr<unsigned>(P.t_nssync) + (size_t)P.g.ns_count() * 32; }
-  // barrier lines and error word start at zero: once per Newton-Schulz phase, in front of its batches
-  void ns_clear_sync() {
-    const long long words = (long long)P.g.ns_count() * 32 + 32;
-    LACT_LAUNCH("k_fill_f32", "k_fill_f32", 0.0, k_fill_f32, dim3((unsigned)((words + 255) / 256)), dim3(256), s, scr<float>(P.t_nssync), 0.f, words);
+  // barrier lines and error word start at zero: once per Newton-Schulz phase, by the kernel in front of its batches
+  ClearWords ns_clear() const {
+    ClearWords c;
+    c.ptr = nullptr; c.n = 0;
+    if (P.muon && ns_fused_any()) { c.ptr = scr<unsigned>(P.t_nssync); c.n = P.g.ns_count() * 32 + 32; }
+    return c;
   }
   template <class TS, bool BWD>
   void launch_ns_fused_ts(NsFusedParams p, const NsBatch& B) {
@@ -698,13 +700,14 @@ struct Runner {
         set_tr_term(jobs[2].t[0], h(2), d.dh, hbs(), kc, d.k_ld, d.k_bs);
         dw_slots = token_reduce("update_dw", jobs, T_);
       }
-      if (P.momentum) LACT_LAUNCH("k_momentum_mean", "k_momentum_mean", 0.0, k_momentum_mean, dim3(d.b), dim3(256), s, mom, (long long)d.kv_len, st.start, T_, mbar(u));
+      // the first update has no earlier momentum state to weigh: its mean is never used
+      if (P.momentum && u > 0) LACT_LAUNCH("k_momentum_mean", "k_momentum_mean", 0.0, k_momentum_mean, dim3(d.b), dim3(256), s, mom, (long long)d.kv_len, st.start, T_, mbar(u));
       {
         MomentumPrepParams p;
         memset(&p, 0, sizeof(p));
         p.g = P.g; p.partial = scr<float>(P.t_partial); p.nsplit = dw_slots;
         p.m_prev = (P.momentum && u > 0) ? dsave(u - 1) : nullptr;
-        p.mbar = P.momentum ? mbar(u) : nullptr;
+        p.mbar = (P.momentum && u > 0) ? mbar(u) : nullptr;
         p.d_out = dsave(u);
         p.g16 = P.muon ? g16(u) : nullptr;
         p.ss_part = scr<float>(P.t_ss);
@@ -721,8 +724,8 @@ struct Runner {
         p.xf = scr<float>(P.t_xf[0]); p.xb = xb(u, 0);
         p.u = P.S == 0 ? usave(u) : nullptr;
         p.plain_bf16 = d.ns_mode == LACT_NS_PLAIN_BF16;
+        p.clear = ns_clear();
         LACT_LAUNCH("k_ns_scale", "k_ns_scale", 0.0, (k_ns_scale<TN>), dim3(P.nblk, P.g.ns_count()), dim3(256), s, p);
-        if (ns_fused_any()) ns_clear_sync();
         for (const NsBatch& B : P.nsb) {
           if (ns_fused_ok(B)) {
             if constexpr (kNsBf16) {
@@ -819,10 +822,13 @@ struct Runner {
     long long maxlen = 0;
     int nb;
     hipStream_t s;
+    bool launched = false;
     ZeroList(int nb_, hipStream_t s_) : nb(nb_), s(s_) {}
     void flush() {
-      if (n > 0 && maxlen > 0)
+      if (n > 0 && maxlen > 0) {
         LACT_LAUNCH("k_zero_segments", "k_zero_segments", 0.0, k_zero_segments, dim3((unsigned)((maxlen + 4095) / 4096), nb, n), dim3(256), s, z);
+        launched = true;
+      }
       n = 0; maxlen = 0;
     }
     void add(void* ptr, long long bs, long long off, long long len) {
@@ -845,25 +851,39 @@ struct Runner {
     float* gmcarry = scr<float>(P.t_gmcarry);
     float* partial = scr<float>(P.t_partial);
     const long long gn0_n = (long long)3 * d.b * P.g.maxrows();
-    LACT_LAUNCH("k_fill_f32", "k_fill_f32", 0.0, k_fill_f32, dim3((unsigned)((gn0_n + 255) / 256)), dim3(256), s, gn0, 0.f, gn0_n);
+    // gn0 is written (not added to) by the first renorm backward; without any update the final kernel reads zeros
+    bool gn0_written = false;
+    if (P.nupd == 0) LACT_LAUNCH("k_fill_f32", "k_fill_f32", 0.0, k_fill_f32, dim3((unsigned)((gn0_n + 255) / 256)), dim3(256), s, gn0, 0.f, gn0_n);
     // gwcur: gradient w.r.t. the current weight version; "not valid" stands for zero (nothing written yet)
     bool gw_valid = dwf && (dwf[0] || dwf[1] || dwf[2]);
     if (gw_valid) LACT_LAUNCH("k_pack3", "k_pack3", 0.0, k_pack3, eg, dim3(256), s, gwcur, P.g.elems, d.b, dwf[0], dwf[1], dwf[2]);
     // every gradient output is written in full by this call: rows that no step touches are zeroed here
+    // The small per-token arrays are added to by the steps, so they are cleared up front on the caller's stream.
+    // Rows of dq, dk, dv that no step writes are disjoint from everything the steps write: nothing waits for
+    // them, and they are cleared on the side stream -- unless ranges overlap partially, where the whole buffers
+    // start at zero and every step adds.
     Touched seen_q, seen_kv;
-    {
-      ZeroList zl(d.b, s);
+    const auto gaps_q = untouched(P.steps, LACT_APPLY, d.q_len, &seen_q.force);
+    const auto gaps_kv = untouched(P.steps, LACT_UPDATE, d.kv_len, &seen_kv.force);
+    const bool rows_on_side = !seen_q.force && !seen_kv.force && s_side != s_main;
+    auto zero_rows = [&](hipStream_t zs) {
+      ZeroList zl(d.b, zs);
       const long long rowb = (long long)d.d * sizeof(T);
-      for (auto& gp : untouched(P.steps, LACT_APPLY, d.q_len, &seen_q.force))
-        zl.add(dq, (long long)d.q_len * rowb, gp.first * rowb, (gp.second - gp.first) * rowb);
-      for (auto& gp : untouched(P.steps, LACT_UPDATE, d.kv_len, &seen_kv.force)) {
+      for (auto& gp : gaps_q) zl.add(dq, (long long)d.q_len * rowb, gp.first * rowb, (gp.second - gp.first) * rowb);
+      for (auto& gp : gaps_kv) {
         zl.add(dk, (long long)d.kv_len * rowb, gp.first * rowb, (gp.second - gp.first) * rowb);
         zl.add(dv, (long long)d.kv_len * rowb, gp.first * rowb, (gp.second - gp.first) * rowb);
       }
+      zl.flush();
+      return zl.launched;
+    };
+    {
+      ZeroList zl(d.b, s);
       float* small[4] = {dlr0, dlr1, dlr2, dmom};
       for (float* ptr : small) zl.add(ptr, (long long)d.kv_len * 4, 0, (long long)d.kv_len * 4);
       zl.flush();
     }
+    if (!rows_on_side) zero_rows(s_main);
     // The apply steps run on the side stream.  Their weight gradients go to gw_side[version & 1] and are added
     // by the consumer of that version's gradient (the renorm backward of the update that made the version, or
     // the final kernel); `free_ev` orders the reuse of a gw_side buffer after its consumer.
@@ -873,6 +893,7 @@ struct Runner {
     hipEvent_t free_ev[2] = {nullptr, nullptr};
     hipEvent_t dw_done[2] = {nullptr, nullptr};   // newest weight-gradient kernel of the apply steps per buffer
     bool side_used = false;
+    if (rows_on_side && zero_rows(s_side)) side_used = true;
     hipEvent_t main_dq_ev = nullptr;   // a dq GEMM on the side stream still reads the main chain's intermediates
     auto wait_main_dq = [&]() {
       if (main_dq_ev) (void)hipStreamWaitEvent(s_main, main_dq_ev, 0);
@@ -967,7 +988,9 @@ struct Runner {
         }
         p.carry_in = (d.prenorm && carry_main >= 0) ? scr<float>(P.t_gwhat[carry_main]) : nullptr;
         p.gw_hat = gwhat;
-        p.gn0 = gn0;
+        p.gn0 = gn0; p.gn0_init = !gn0_written;
+        gn0_written = true;
+        p.clear = ns_clear();
         if (P.muon) { p.gxf = scr<float>(P.t_gxf[0]); p.gxb = scr<TN>(P.t_gxb[0]); }
         LACT_LAUNCH("k_renorm_bwd", "k_renorm_bwd", 0.0, (k_renorm_bwd<TN>), rowgrid, dim3(256), s, p);
         if (side_valid[sb]) {
@@ -980,7 +1003,6 @@ struct Runner {
       }
       if (d.prenorm) carry_main = gw_idx;
       if (P.muon) {
-        if (ns_fused_any()) ns_clear_sync();
         for (const NsBatch& B : P.nsb) {
           const int n = B.n, r = B.r, c = B.c;
           const long long xe = (long long)r * c, se = (long long)r * r;
@@ -1047,9 +1069,10 @@ struct Runner {
         p.gx0 = scr<float>(P.t_gxf[cur]); p.g16 = P.muon ? (const void*)g16(u) : nullptr; p.norms = norms(u);
         p.dot_part = scr<float>(P.t_dot); p.nparts = P.nblk;
         p.gw_hat = gwhat; p.cr = (P.muon && d.muon_replaces_weight) ? 1.f : 0.f;
-        p.gm_carry = P.momentum ? gmcarry : nullptr; p.carry_valid = gm_valid;
+        p.gm_carry = (P.momentum && (u > 0 || gm_valid)) ? gmcarry : nullptr; p.carry_valid = gm_valid;
+        p.carry_write = u > 0;
         p.m_prev = (P.momentum && u > 0) ? dsave(u - 1) : nullptr;
-        p.mbar = P.momentum ? mbar(u) : nullptr;
+        p.mbar = (P.momentum && u > 0) ? mbar(u) : nullptr;
         p.gc = scr<T>(P.t_gc);
         p.mdot_part = scr<float>(P.t_mdot);
         if (P.muon && ns_fused_any()) p.poison = ns_error_word();

@@ -95,6 +95,16 @@ __global__ void k_init_state(const InitParams p) {
   if (lane == 0) p.n0[(size_t)z * p.g.maxrows() + row] = sqrtf(ss);
 }
 
+// Side job of a kernel that runs right before a fused Newton-Schulz launch: its first block clears the barrier
+// lines and the error word (a few KiB), which saves a launch of its own in the dependent chain.
+struct ClearWords {
+  unsigned* ptr; int n;
+};
+__device__ __forceinline__ void clear_words(const ClearWords& c, bool first_block) {
+  if (c.n > 0 && first_block)
+    for (int i = threadIdx.x; i < c.n; i += blockDim.x) c.ptr[i] = 0u;
+}
+
 // ---- mean of the per-token momentum over one chunk (ttt_operation.py:171-172) --------------------
 __global__ void k_momentum_mean(const float* mom, long long bs, int start, int len, float* mbar) {
   __shared__ float red[16];
@@ -167,11 +177,13 @@ struct NsScaleParams {
   float* xf; void* xb;   // [3b][elems], Newton-Schulz orientation (fp32 iterate, copy in the Newton-Schulz type)
   float* u;              // [3b][elems] original orientation, or null (only when zero iterations follow)
   int plain_bf16;        // reference without autocast: norm and quotient are bf16 tensors
+  ClearWords clear;
 };
 // Grid (chunks, Newton-Schulz matrices).  ss_part is indexed by packed matrix.
 template <typename TN>
 __global__ void k_ns_scale(const NsScaleParams p) {
   const int m = blockIdx.y;
+  clear_words(p.clear, blockIdx.x == 0 && blockIdx.y == 0);
   float ss = 0.f;
   for (int i = 0; i < p.nparts; ++i) ss += p.ss_part[(size_t)p.g.ns_part0(m) * p.nparts + i];
   if (p.g.ns_part1(m) >= 0)
@@ -228,7 +240,9 @@ struct RenormParams {
   const float* gy2;                // second addend of the same gradient (the apply steps' share), or null
   const float* carry_in;           // gradient arriving at the accumulator from later steps (pre-norm) or null
   float* gw_hat;                   // gradient w.r.t. w_hat, original orientation
-  float* gn0;                      // [3b][maxrows], accumulated
+  float* gn0;                      // [3b][maxrows], accumulated (written when gn0_init: first use in a backward pass)
+  int gn0_init;
+  ClearWords clear;
   float* gxf; void* gxb;           // the same gradient in Newton-Schulz orientation (fp32 + Newton-Schulz type) or null
 };
 // off: offset in the packed arrays; uo: offset of the same element in `u`
@@ -305,6 +319,7 @@ template <typename TN>
 __global__ void k_renorm_bwd(const RenormParams p) {
   const int z = blockIdx.y, j = z / p.g.nb;
   const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  clear_words(p.clear, blockIdx.x == 0 && blockIdx.y == 0);
   if (row >= p.g.rows(j)) return;
   const int cols = p.g.cols(j);
   const size_t o = (size_t)z * p.g.elems + (size_t)row * cols;
@@ -312,6 +327,8 @@ __global__ void k_renorm_bwd(const RenormParams p) {
   const size_t xo = p.g.ns_base(p.g.ns_of(z));
   const bool contiguous = p.g.x_contiguous(j);
   float c0 = 1.f, c1 = 0.f;
+  float* gn0 = p.gn0 + (size_t)z * p.g.maxrows() + row;
+  if (!p.weight_norm && p.gn0_init && lane == 0) *gn0 = 0.f;
   if (p.weight_norm) {
     float ss = 0.f, dot = 0.f;
     for (int c = lane * 4; c < cols; c += 256) {
@@ -326,12 +343,12 @@ __global__ void k_renorm_bwd(const RenormParams p) {
       const float den = sqrtf(ss + 1e-5f);
       c0 = n0 / den;
       c1 = dot * n0 / (den * den * den);
-      if (lane == 0) p.gn0[(size_t)z * p.g.maxrows() + row] += dot / den;
+      if (lane == 0) *gn0 = (p.gn0_init ? 0.f : *gn0) + dot / den;
     } else {               // den = r + eps:  d den / d w = w / r
       const float r = sqrtf(ss);
       c0 = n0 / (r + 1e-5f);
       c1 = r > 0.f ? dot * n0 / (r * (r + 1e-5f) * (r + 1e-5f)) : 0.f;
-      if (lane == 0) p.gn0[(size_t)z * p.g.maxrows() + row] += dot / (r + 1e-5f);
+      if (lane == 0) *gn0 = (p.gn0_init ? 0.f : *gn0) + dot / (r + 1e-5f);
     }
   }
   for (int c = lane * 4; c < cols; c += 256) {
@@ -393,6 +410,7 @@ struct GradPrepParams {
   const float* gx0; const void* g16; const float* norms; const float* dot_part; int nparts;
   const float* gw_hat; float cr;     // added when the raw gradient also enters w_hat
   float* gm_carry; int carry_valid;  // gradient w.r.t. the momentum state after this update (in/out)
+  int carry_write;                   // an earlier update exists: hand it gm_carry = g * mbar
   const float* m_prev; const float* mbar;   // null without momentum
   void* gc;                          // [3b][elems] compute-type copy of d loss / d dw  (GEMM operand)
   float* mdot_part;                  // [3b][gridDim.x] partial <g, m_prev>
@@ -451,12 +469,12 @@ __global__ void k_grad_prep(const GradPrepParams p) {
         const float4 cv = ld4(p.gm_carry + o);
         gv.x += cv.x; gv.y += cv.y; gv.z += cv.z; gv.w += cv.w;
       }
-      st4(p.gm_carry + o, f4(gv.x * mb, gv.y * mb, gv.z * mb, gv.w * mb));   // d/d M_prev of  dw + M_prev * mbar
+      if (p.carry_write) st4(p.gm_carry + o, f4(gv.x * mb, gv.y * mb, gv.z * mb, gv.w * mb));   // d/d M_prev of  dw + M_prev * mbar
       if (p.m_prev) md += dot4(gv, ld4(p.m_prev + o));
     }
     Elem<T>::store4(reinterpret_cast<T*>(p.gc) + o, gv.x, gv.y, gv.z, gv.w);
   }
-  if (p.gm_carry) {
+  if (p.gm_carry && p.m_prev) {
     md = block_sum(md, red);
     if (threadIdx.x == 0) p.mdot_part[(size_t)z * gridDim.x + blockIdx.x] = md;
   }
