@@ -143,9 +143,10 @@ int lact_layer_post_backward(int32_t act_dtype, int32_t B, int32_t L, int32_t H,
 /* Execution options (process-wide; no counterpart in the reference, where PyTorch enqueues the whole layer on one
  * stream as separate kernels).  Both are on by default and change no result bit.
  *   LACT_OPT_STREAM_OVERLAP: the apply steps of a program do not depend on the update chain that runs beside
- *     them; lact_forward / lact_backward enqueue them on a library-owned second stream (default priority, one
- *     per device, created on first use) that is forked from and joined back into the caller's stream with
- *     events, so the call as a whole stays asynchronous and ordered on the caller's stream.
+ *     them, and nothing in a call waits for dk, dv or the learning-rate gradients of an update; lact_forward /
+ *     lact_backward enqueue them on two library-owned streams (default priority, per device, created on first
+ *     use) that are forked from and joined back into the caller's stream with events, so the call as a whole
+ *     stays asynchronous and ordered on the caller's stream.
  *   LACT_OPT_FUSED_NEWTON_SCHULZ: all Newton-Schulz iterations of an update (and of its backward) run as one
  *     kernel whose blocks meet at per-matrix barriers (bf16, rows and columns multiples of 192 or of 128, at most 8
  *     iterations); otherwise three GEMM launches per iteration.

@@ -58,7 +58,9 @@ template <> struct Elem<float> {
   }
 };
 
-__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
+// one v_exp_f32 and one v_rcp_f32 (1 ulp) instead of the ten-instruction IEEE division: the epilogues that call
+// this per element are bound by vector-ALU issue
+__device__ __forceinline__ float sigmoidf_(float x) { return __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
 
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -4,6 +4,7 @@
 #include "../../include/lact_hip.h"
 
 #include <algorithm>
+#include <atomic>
 #include <cstdio>
 #include <cstring>
 #include <string>
@@ -85,11 +86,21 @@ struct ProfScope {
     hipLaunchKernelGGL(kern, grid, block, smem_bytes, stream, __VA_ARGS__);              \
   } while (0)
 
-// kernels whose ring exceeds the default dynamic LDS limit opt in once per instantiation
-template <class K>
-void allow_big_lds(K kern, int bytes) {
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+// Kernels whose ring exceeds the default dynamic LDS limit opt in once per call site (= instantiation) and device:
+// the attribute belongs to the current device.
+inline void allow_big_lds(std::atomic<uint64_t>& done, const void* kern, int bytes) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+  const uint64_t bit = 1ull << dev;
+  if (done.load(std::memory_order_acquire) & bit) return;
+  (void)hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  done.fetch_or(bit, std::memory_order_release);
 }
+#define LACT_BIG_LDS(kern, bytes)                                         \
+  do {                                                                    \
+    static std::atomic<uint64_t> done_{0};                                \
+    allow_big_lds(done_, reinterpret_cast<const void*>(kern), bytes);     \
+  } while (0)
 
 template <typename T> const char* tname();
 template <> const char* tname<uint16_t>() { return "bf16"; }
@@ -108,6 +119,7 @@ template <> const char* tname<float>() { return "f32"; }
 // pool per device, created on first use and kept until the process ends.
 struct SideCtx {
   hipStream_t stream = nullptr;
+  hipStream_t tail = nullptr;        // second side stream: results of the update chain that nothing in the call waits for
   std::vector<hipEvent_t> ev;
   size_t next = 0;
   hipEvent_t fused_done = nullptr;   // completion of the newest fused Newton-Schulz kernel of this process
@@ -130,6 +142,7 @@ SideCtx* side_ctx() {
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
   SideCtx& c = ctx[dev];
   if (!c.stream && hipStreamCreateWithFlags(&c.stream, hipStreamNonBlocking) != hipSuccess) return nullptr;
+  if (!c.tail && hipStreamCreateWithFlags(&c.tail, hipStreamNonBlocking) != hipSuccess) return nullptr;
   c.next = 0;
   return &c;
 }
@@ -315,8 +328,7 @@ template <class TS, int NT, int EPI, bool B_KS>
 void launch_row_gemm_dma(const char* site, const RowGemmDmaParams<NT>& q, int batch, hipStream_t s) {
   constexpr int STAGES = row_stages<TS>();
   constexpr int SMEM = cmax(DmaSmem<TS, 1, STAGES>::BYTES, StageTile<TS, 4>::BYTES);
-  static bool once = (allow_big_lds(k_row_gemm_dma<TS, NT, EPI, B_KS>, SMEM), true);
-  (void)once;
+  LACT_BIG_LDS((k_row_gemm_dma<TS, NT, EPI, B_KS>), SMEM);
   static const std::string name = std::string("k_row_gemm_dma<") + std::to_string(TS::BM) + "x" + std::to_string(TS::BN) + "," +
                                   std::to_string(NT) + (EPI == EPI_STORE ? ",store" : (EPI == EPI_AXPBY ? ",axpby" : ",axpby_dual")) +
                                   (B_KS ? ",Bks>" : ",Bkc>");
@@ -411,13 +423,14 @@ struct Runner {
   char* sc;   // scratch
   const lact_desc_t& d;
   hipStream_t s_main, s_side;   // caller's stream; stream of the apply steps (= s_main when overlap is off)
+  hipStream_t s_tail;           // stream of dk, dv and the learning-rate gradients (= s_main when overlap is off)
   SideCtx* side = nullptr;
   const size_t* hsel;           // token-major intermediates of the chain being enqueued
   size_t partial_sel;
   Runner(const Plan& p, void* saved, void* scratch, hipStream_t st)
-      : P(p), s(st), sv(align256(saved)), sc(align256(scratch)), d(p.d), s_main(st), s_side(st), hsel(p.t_h), partial_sel(p.t_partial) {
+      : P(p), s(st), sv(align256(saved)), sc(align256(scratch)), d(p.d), s_main(st), s_side(st), s_tail(st), hsel(p.t_h), partial_sel(p.t_partial) {
     side = side_ctx();
-    if (side && g_overlap) s_side = side->stream;
+    if (side && g_overlap) { s_side = side->stream; s_tail = side->tail; }
   }
   // ---- fused Newton-Schulz: launches of at most 256 resident blocks
   static bool tiles_fit(int r, int c, int edge) { return r % edge == 0 && c % edge == 0 && (r / edge) * (c / edge) <= 32; }
@@ -447,8 +460,7 @@ struct Runner {
   template <class TS, bool BWD>
   void launch_ns_fused_ts(NsFusedParams p, const NsBatch& B) {
     constexpr int SM = cmax(DmaSmem<TS, 1, row_stages<TS>()>::BYTES, StageTile<TS, 4>::BYTES);
-    static bool once = (allow_big_lds(k_ns_fused<TS, BWD>, SM), true);
-    (void)once;
+    LACT_BIG_LDS((k_ns_fused<TS, BWD>), SM);
     const int nbm = (B.r / TS::BM) * (B.c / TS::BN);
     const int per = (256 / nbm) / 8 * 8;
     unsigned* sync = scr<unsigned>(P.t_nssync) + (size_t)B.first * 32;
@@ -520,9 +532,10 @@ struct Runner {
       const TileMap m6 = make_tile_map(ceil_div(T_, TS_BWD::BM), ceil_div(d.dh, TS_BWD::BN), d.b);
       q.map = which == 3 ? m6 : m3;
       dim3 g3(m3.grid()), g6(m6.grid());
-      static bool once = (allow_big_lds(k_apply_hidden_dma<TS_SQ>, SM3), allow_big_lds(k_update_hidden_dma<TS_SQ>, SM3),
-                          allow_big_lds(k_apply_bwd_hidden_dma<TS_SQ>, SM3), allow_big_lds(k_update_bwd_hidden_dma<TS_BWD>, SM6), true);
-      (void)once;
+      LACT_BIG_LDS(k_apply_hidden_dma<TS_SQ>, SM3);
+      LACT_BIG_LDS(k_update_hidden_dma<TS_SQ>, SM3);
+      LACT_BIG_LDS(k_apply_bwd_hidden_dma<TS_SQ>, SM3);
+      LACT_BIG_LDS(k_update_bwd_hidden_dma<TS_BWD>, SM6);
       if (which == 0) LACT_LAUNCH_SMEM("k_apply_hidden_dma", "apply_hidden", 4.0 * f, (k_apply_hidden_dma<TS_SQ>), g3, dim3(DMA_THREADS), SM3, s, q);
       if (which == 1) LACT_LAUNCH_SMEM("k_update_hidden_dma", "update_hidden", 6.0 * f, (k_update_hidden_dma<TS_SQ>), g3, dim3(DMA_THREADS), SM3, s, q);
       if (which == 2) LACT_LAUNCH_SMEM("k_apply_bwd_hidden_dma", "apply_bwd_hidden", 6.0 * f, (k_apply_bwd_hidden_dma<TS_SQ>), g3, dim3(DMA_THREADS), SM3, s, q);
@@ -583,13 +596,11 @@ struct Runner {
         else slots = sp.n;
         if (big) {
           constexpr int SM = cmax(DmaSmem<TS_NS, 1, row_stages<TS_NS>()>::BYTES, StageTile<TS_NS, 4>::BYTES);
-          static bool once = (allow_big_lds(k_token_reduce_dma<TS_NS>, SM), true);
-          (void)once;
+          LACT_BIG_LDS(k_token_reduce_dma<TS_NS>, SM);
           LACT_LAUNCH_SMEM("k_token_reduce_dma<192x192>", site, fl, (k_token_reduce_dma<TS_NS>), g, dim3(DMA_THREADS), SM, s, pd);
         } else {
           constexpr int SM = cmax(DmaSmem<TS_SQ, 1, row_stages<TS_SQ>()>::BYTES, StageTile<TS_SQ, 4>::BYTES);
-          static bool once = (allow_big_lds(k_token_reduce_dma<TS_SQ>, SM), true);
-          (void)once;
+          LACT_BIG_LDS(k_token_reduce_dma<TS_SQ>, SM);
           LACT_LAUNCH_SMEM("k_token_reduce_dma<128x128>", site, fl, (k_token_reduce_dma<TS_SQ>), g, dim3(DMA_THREADS), SM, s, pd);
         }
         if (main_tokens == tokens) return slots;
@@ -899,6 +910,15 @@ struct Runner {
       if (main_dq_ev) (void)hipStreamWaitEvent(s_main, main_dq_ev, 0);
       main_dq_ev = nullptr;
     };
+    // dk, dv and the learning-rate gradients of an update: nothing in the call waits for them, so they run on the
+    // tail stream beside the rest of the chain.  They read the chain's token-major intermediates, the compute-type
+    // gradient copy and the row partials: the chain waits for `tail_ev` before it writes any of those again.
+    hipEvent_t tail_ev = nullptr;
+    bool tail_used = false;
+    auto wait_tail = [&]() {
+      if (tail_ev) (void)hipStreamWaitEvent(s_main, tail_ev, 0);
+      tail_ev = nullptr;
+    };
     float* partial_side = scr<float>(P.t_partial_side);
     int ver = P.nupd, u = P.nupd;
     int carry_main = -1;       // index of the gwhat buffer holding the accumulator's gradient (pre-norm)
@@ -932,6 +952,7 @@ struct Runner {
           // so they stay on the caller's stream (no event hand-over in the critical path); only dq, which nothing
           // waits for, goes to the side stream and reads this chain's intermediates.
           wait_main_dq();
+          wait_tail();
           HiddenParams hp = hidden_params(T_, qc, d.q_ld, d.q_bs, gc, d.do_ld, d.do_bs, ver);
           hp.O0 = h(0); hp.O1 = h(1); hp.O2 = h(2);
           launch_hidden(2, hp, ver, T_);
@@ -1063,6 +1084,7 @@ struct Runner {
         LACT_LAUNCH("k_ns_bwd_dot", "k_ns_bwd_dot", 0.0, (k_ns_bwd_dot<TN>), dim3(P.nblk, P.g.ns_count()), dim3(256), s, dp);
       }
       {
+        wait_tail();   // the previous update's dk GEMM reads the gradient copy written here
         GradPrepParams p;
         memset(&p, 0, sizeof(p));
         p.g = P.g; p.muon = P.muon;
@@ -1097,9 +1119,16 @@ struct Runner {
         hp.lrpart_stride = (long long)d.b * P.Tcap;
         hp.lrpart_mat_stride = (long long)P.lr_slots * d.b * P.Tcap;
         wait_main_dq();
+        wait_tail();
         launch_hidden(3, hp, vprev, T_);
       }
       const bool acc_kv = seen_kv.accumulate(st.start, st.end);
+      // worth a hand-over only when an earlier update's chain follows on the caller's stream
+      const bool use_tail = s_tail != s_main && u > 0;
+      if (use_tail) {
+        wait_for(s_tail, s_main);
+        s = s_tail;
+      }
       {  // dk = (dgate*lr0) G0 + (dh2*lr2) G2 + gG W0 + gH2 W2
         auto p = row_params<4>();
         set_term(p.t[0], h(3), d.dh, hbs(), g0, d.d, P.g.elems, d.dh);
@@ -1118,6 +1147,16 @@ struct Runner {
         p.accumulate = acc_kv;
         launch_row_gemm<T, true, 2, EPI_STORE>("update_bwd_dv", p, d.b, s, true);
       }
+      LACT_LAUNCH("k_lr_reduce", "k_lr_reduce", 0.0, k_lr_reduce, dim3(ceil_div(T_, 256), d.b, 3), dim3(256), s, scr<float>(P.t_lrpart),
+                         (long long)P.lr_slots * d.b * P.Tcap, (long long)d.b * P.Tcap,
+                  kBf16 ? ceil_div(d.dh, TS_BWD::BN) * TS_BWD::WAVES_N : ceil_div(d.dh, TSB::BN) * TSB::WAVES_N, P.Tcap, dlr0, dlr1, dlr2,
+                         (long long)d.kv_len, st.start, T_);
+      if (use_tail) {
+        s = s_main;
+        tail_ev = side->event();
+        (void)hipEventRecord(tail_ev, s_tail);
+        tail_used = true;
+      }
       {
         TokenReduceJob jobs[3];
         memset(jobs, 0, sizeof(jobs));
@@ -1133,15 +1172,12 @@ struct Runner {
           LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, gwcur, pass != 0.f ? gwhat : nullptr, pass, partial, ns_, (long long)P.mat3);
         gw_valid = true;
       }
-      LACT_LAUNCH("k_lr_reduce", "k_lr_reduce", 0.0, k_lr_reduce, dim3(ceil_div(T_, 256), d.b, 3), dim3(256), s, scr<float>(P.t_lrpart),
-                         (long long)P.lr_slots * d.b * P.Tcap, (long long)d.b * P.Tcap,
-                  kBf16 ? ceil_div(d.dh, TS_BWD::BN) * TS_BWD::WAVES_N : ceil_div(d.dh, TSB::BN) * TSB::WAVES_N, P.Tcap, dlr0, dlr1, dlr2,
-                         (long long)d.kv_len, st.start, T_);
       --ver;
     }
     {
       FinishParams p;
       if (side_used) wait_for(s_main, s_side);
+      if (tail_used) wait_tail();
       p.g = P.g; p.gw = gw_valid ? gwcur : nullptr;
       p.gw2 = side_valid[0] ? gw_side[0] : nullptr;
       p.carry = (d.prenorm && carry_main >= 0) ? scr<float>(P.t_gwhat[carry_main]) : nullptr;
