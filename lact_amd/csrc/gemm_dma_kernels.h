@@ -9,7 +9,7 @@ namespace lact {
 
 using TS_ROW = TileShape<256, 128, 2, 2>;   // token-row GEMMs, one accumulator: 128x64 per wave
 using TS_SQ = TileShape<128, 128, 2, 2>;    // small square GEMMs (Newton-Schulz) and 2-3 accumulator kernels
-using TS_BWD = TileShape<64, 128, 1, 4>;    // six accumulators (update backward): 64x32 per wave
+using TS_BWD = TileShape<128, 64, 2, 2>;    // six accumulators (update backward): 64x32 per wave
 using TS_NS = TileShape<192, 192, 2, 2>;    // 384-multiple square GEMMs (Newton-Schulz at d = dh = 384): 96x96 per wave
 
 template <class TS> constexpr int row_stages() { return TS::BM == 128 ? 4 : 3; }
