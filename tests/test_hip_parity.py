@@ -400,15 +400,11 @@ def test_ar_video_inference_repeat_accumulates_kv_grads():
 
 
 # ---- size-independent properties at the benchmark size ----------------------------------------------
-def test_config1_full_size_properties():
-    """BASELINE config 1 (b=16, L=4096, d=dh=384, chunk 2048, Muon, momentum 0.9, fwd+bwd) at full size:
-    determinism, block causality, head independence -- bit-exact checks no oracle run is needed for --
-    plus the first chunk against the oracle (its output does not depend on any update)."""
-    say("config 1 full-size properties")
-    b, L, d, dh, C = 16, 4096, 384, 384, 2048
-    inp = O.make_inputs(b, L, d, dh, seed=1001, act_dtype=torch.bfloat16, distinct_heads=4)
+def full_size_properties(b, L, d, dh, C, seed, single_update):
+    inp = O.make_inputs(b, L, d, dh, seed=seed, act_dtype=torch.bfloat16, distinct_heads=4)
     g = clone_to(inp, DEV)
     go = torch.randn(b, L, d, generator=torch.Generator().manual_seed(3)).bfloat16().to(DEV)
+    last = ((L - 1) // C) * C        # first row of the last chunk
 
     def run(t, upstream=None):
         out = T.block_causal_lact_swiglu(*args9(t), C, True, t["momentum"])
@@ -420,24 +416,49 @@ def test_config1_full_size_properties():
     ref0 = O.swiglu_apply(inp["w0"], inp["w1"], inp["w2"], inp["q"][:, :C], AC)
     assert O.rel_l2(out1[:, :C], ref0) < 1e-3
     # causality: k, v of the last chunk are never read; their gradients are exactly zero
-    assert float(gr1["k"][:, C:].abs().max()) == 0.0 and float(gr1["v"][:, C:].abs().max()) == 0.0
-    assert float(gr1["lr0"][:, C:].abs().max()) == 0.0 and float(gr1["momentum"][:, C:].abs().max()) == 0.0
+    assert float(gr1["k"][:, last:].abs().max()) == 0.0 and float(gr1["v"][:, last:].abs().max()) == 0.0
+    assert float(gr1["lr0"][:, last:].abs().max()) == 0.0 and float(gr1["momentum"][:, last:].abs().max()) == 0.0
     t2 = clone_to(inp, DEV)
     with torch.no_grad():
-        t2["k"][:, C + 5] += 1.0
-        t2["v"][:, C + 7] -= 1.0
-        t2["q"][:, C + 9] += 1.0                                       # only row C+9 of the output may move
+        t2["k"][:, last + 5] += 1.0
+        t2["v"][:, last + 7] -= 1.0
+        t2["q"][:, last + 9] += 1.0                                    # only row last+9 of the output may move
     out3, _ = run(t2)
-    assert torch.equal(out3[:, :C], out1[:, :C])
-    keep = torch.ones(L, dtype=torch.bool); keep[C + 9] = False
+    keep = torch.ones(L, dtype=torch.bool); keep[last + 9] = False
     assert torch.equal(out3[:, keep.to(DEV)], out1[:, keep.to(DEV)])
+    assert not torch.equal(out3[:, last + 9], out1[:, last + 9])
     # heads never interact: a permutation of the batch permutes outputs and gradients bit-exactly
     perm = torch.randperm(b, generator=torch.Generator().manual_seed(1)).to(DEV)
     t3 = {n: (None if v is None else v.detach()[perm].clone().requires_grad_(True)) for n, v in g.items()}
     out4, gr4 = run(t3, go[perm])
     assert torch.equal(out4, out1[perm]) and torch.equal(gr4["w1"], gr1["w1"][perm]) and torch.equal(gr4["k"], gr1["k"][perm])
-    # with momentum == 0 after the only update nothing is carried: d loss / d momentum is <g, M_prev> = 0
-    assert float(gr1["momentum"].abs().max()) == 0.0
+    if single_update:
+        # nothing is carried into the only update: d loss / d momentum is <g, M_prev> = 0
+        assert float(gr1["momentum"].abs().max()) == 0.0
+    else:
+        # the first chunk's momentum weighs no earlier state; later chunks' momentum does
+        assert float(gr1["momentum"][:, :C].abs().max()) == 0.0 and float(gr1["momentum"][:, C:last].abs().max()) > 0.0
+
+
+def test_config1_full_size_properties():
+    """BASELINE config 1 (b=16, L=4096, d=dh=384, chunk 2048, Muon, momentum 0.9, fwd+bwd) at full size:
+    determinism, block causality, head independence -- bit-exact checks no oracle run is needed for --
+    plus the first chunk against the oracle (its output does not depend on any update)."""
+    say("config 1 full-size properties")
+    full_size_properties(16, 4096, 384, 384, 2048, 1001, True)
+
+
+def test_config2_full_size_properties():
+    """BASELINE config 2 (b=4, L=32768, d=dh=384, chunk 2048: 15 chained updates) at full size."""
+    say("config 2 full-size properties")
+    full_size_properties(4, 32768, 384, 384, 2048, 1002, False)
+
+
+def test_config4_full_size_properties():
+    """BASELINE config 4 (b=12, L=32760, d=128, dh=256, chunk 4680 = 73 x 64 + 8 tokens: ragged token tiles) at
+    full size."""
+    say("config 4 full-size properties")
+    full_size_properties(12, 32760, 128, 256, 4680, 1004, False)
 
 
 @pytest.mark.parametrize("prenorm", [False, True])
