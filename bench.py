@@ -28,6 +28,10 @@ CONFIGS = {
            "config 2: block_causal_lact_swiglu fwd+bwd, B=1 H=4 (b=4), L=32768, d=dh=384, chunk 2048, Muon + momentum"),
     "c4": (1, 12, 32760, 128, 256, 4680, 1004,
            "config 4: block_causal_lact_swiglu fwd+bwd, video shape b=12, L=32760, d=128, dh=256, chunk 4680, Muon + momentum"),
+    # forward only: one update on 8192 tokens (8 input views), one apply on 1024 tokens (the target view)
+    "c3": (1, 6, 9216, 128, 256, 8192, 1003,
+           "config 3: fast_weight_swish_glu_weight_norm_mini_batch_apply forward only, NVS shape b=6, d=128, dh=256, "
+           "update on 8192 tokens then apply on 1024, Muon with 5 classic Newton-Schulz steps"),
 }
 
 
@@ -96,6 +100,19 @@ def main():
         out.backward(go)
         return out
 
+    if args.config == "c3":
+        import math as _m
+        from lact_amd import nvs
+        inp3 = O.make_inputs(b, L, d, dh, seed=seed, act_dtype=torch.bfloat16, momentum_value=None)
+        for n in ("w0", "w1", "w2"):      # transposed layout and sqrt(2) gain of lact_nvs/lact_ttt.py:184-193
+            inp3[n] = (inp3[n] * _m.sqrt(2.0)).transpose(1, 2).contiguous()
+        dev3 = [inp3[n].to("cuda:0") for n in order]
+        program = [nvs.TTTOperator(0, C, True, False), nvs.TTTOperator(C, L, False, True)]
+
+        def step():   # noqa: F811
+            with torch.no_grad():
+                return nvs.fast_weight_swish_glu_weight_norm_mini_batch_apply(*dev3, program, 5)[0]
+
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0").random_(0, 255)
         dst = torch.empty_like(src)
@@ -117,6 +134,9 @@ def main():
     ms_per_step = dt / args.steps * 1e3
     tokens_per_s = B * L * args.steps / dt
     flops = algorithmic_flops(b, L, d, dh, C)
+    if args.config == "c3":   # forward only; apply on L - C tokens, one update on C tokens
+        r_, c_ = min(d, dh), max(d, dh)
+        flops = b * (6.0 * d * dh * (L - C) + 12.0 * d * dh * C + 3.0 * 5 * (4.0 * r_ * r_ * c_ + 2.0 * r_ ** 3))
     op_tflops = flops / (ms_per_step * 1e-3) / 1e12
 
     res = {
@@ -171,15 +191,20 @@ def main():
         t0 = time.perf_counter()
         reps = 0
         while reps < 1 or (time.perf_counter() - t0 < 12.0 and reps < 40):
-            for t in cpu.values():
-                t.grad = None
-            o = O.block_causal_lact_swiglu(*[cpu[n] for n in order], C, True, cpu["momentum"], num=O.Numerics(autocast=True))
-            o.backward(gc)
+            if args.config == "c3":   # forward only, as the GPU leg
+                with torch.no_grad():
+                    O.fast_weight_swish_glu_weight_norm_mini_batch_apply(*[inp3[n][:cb] for n in order], program, 5,
+                                                                         num=O.Numerics(autocast=True))
+            else:
+                for t in cpu.values():
+                    t.grad = None
+                o = O.block_causal_lact_swiglu(*[cpu[n] for n in order], C, True, cpu["momentum"], num=O.Numerics(autocast=True))
+                o.backward(gc)
             reps += 1
         ct = (time.perf_counter() - t0) / reps
         res["cpu_baseline"] = {"value": (B * L) * (cb / b) / ct, "unit": "tokens/s", "cores": torch.get_num_threads(),
                                "kind": "port",
-                               "sample": f"first {cb} of {b} heads of the same workload, fwd+bwd, {reps} run(s), "
+                               "sample": f"first {cb} of {b} heads of the same workload, {'fwd' if args.config == 'c3' else 'fwd+bwd'}, {reps} run(s), "
                                          f"{ct:.2f} s each; tokens scaled by {cb}/{b}; host has {os.cpu_count()} logical CPUs"}
     print(json.dumps(res))
 
