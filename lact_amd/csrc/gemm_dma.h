@@ -368,6 +368,10 @@ struct StageTile {
     if (E == 2) Elem<uint16_t>::store4(reinterpret_cast<uint16_t*>(base + frag_off(tm, tn, g)), a, b, c, d);
     else *reinterpret_cast<float4*>(base + frag_off(tm, tn, g)) = make_float4(a, b, c, d);
   }
+  __device__ static __forceinline__ void get4(const char* base, int tm, int tn, int g, float (&o)[4]) {
+    static_assert(E == 2, "staged inputs are bf16 tiles");
+    Elem<uint16_t>::load4(reinterpret_cast<const uint16_t*>(base + frag_off(tm, tn, g)), o);
+  }
   // this thread's position in the copy-out phase
   __device__ static __forceinline__ bool active() { return (int)threadIdx.x < RPP * LPR; }   // RPP*LPR <= 256: loader wave idle
   __device__ static __forceinline__ int row0() { return threadIdx.x / LPR; }

@@ -360,6 +360,25 @@ __global__ __launch_bounds__(DMA_THREADS) void k_update_hidden_dma(const HiddenD
   copy_out_b16<TS>(smem + 0 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O0) + off, p.dh, p.T - m0, p.dh - n0);
   copy_out_b16<TS>(smem + 1 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O1) + off, p.dh, p.T - m0, p.dh - n0);
   copy_out_b16<TS>(smem + 2 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O2) + off, p.dh, p.T - m0, p.dh - n0);
+  if (p.O3) {   // the backward is going to start from the rounded pre-activations instead of recomputing them
+    __syncthreads();
+#pragma unroll
+    for (int tm = 0; tm < TS::TM; ++tm) {
+      if (tm >= ntm) break;
+#pragma unroll
+      for (int tn = 0; tn < TS::TN; ++tn)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          SB::put4(s0, tm, tn, g, a02[0][tm][tn][4 * g], a02[0][tm][tn][4 * g + 1], a02[0][tm][tn][4 * g + 2], a02[0][tm][tn][4 * g + 3]);
+          SB::put4(s1, tm, tn, g, a02[1][tm][tn][4 * g], a02[1][tm][tn][4 * g + 1], a02[1][tm][tn][4 * g + 2], a02[1][tm][tn][4 * g + 3]);
+          SB::put4(s2, tm, tn, g, a1[0][tm][tn][4 * g], a1[0][tm][tn][4 * g + 1], a1[0][tm][tn][4 * g + 2], a1[0][tm][tn][4 * g + 3]);
+        }
+    }
+    __syncthreads();
+    copy_out_b16<TS>(smem + 0 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O3) + off, p.dh, p.T - m0, p.dh - n0);
+    copy_out_b16<TS>(smem + 1 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O4) + off, p.dh, p.T - m0, p.dh - n0);
+    copy_out_b16<TS>(smem + 2 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O5) + off, p.dh, p.T - m0, p.dh - n0);
+  }
 }
 
 template <class TS>
@@ -480,6 +499,148 @@ __global__ __launch_bounds__(DMA_THREADS) void k_update_bwd_hidden_dma(const Hid
 #pragma unroll
   for (int i = 0; i < 6; ++i)
     copy_out_b16<TS>(smem + i * SB::BYTES, reinterpret_cast<uint16_t*>(outs[i]) + off, p.dh, p.T - m0, p.dh - n0);
+}
+
+// update backward, hidden stage, from the pre-activations the forward kept (I0 = k W0^T, I1 = k W2^T, I2 = v W1,
+// rounded as the forward rounded them): only the three products with the gradient matrices are left,
+// phases (X; G0, G2) and (Y; G1 read K-strided).  O0..O2 as in k_update_bwd_hidden_dma; what that kernel writes
+// to O3..O5 are the forward's own lr-scaled operands, which the forward kept as well.
+// The block's three input tiles travel through the ring like operands: a last phase of one or two K-steps copies
+// columns [64h, 64h + 64) of I0, I1, I2 into the A, B0, B1 places of a stage, where they simply stay -- the matrix
+// waves only pass the barriers of those K-steps.  Every lane then finds the inputs of its accumulator positions
+// in those stages (same swizzle as any operand tile), overwrites them with the results, and the block copies the
+// stages out.  dh must be a multiple of 64.
+template <class TS>
+__global__ __launch_bounds__(DMA_THREADS) void k_update_bwd_hidden_kept_dma(const HiddenDmaParams pp) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  static_assert(TS::BM == 128 && TS::BN == 128 && TS::WN == 64, "one wave column per 64-column half of the tile");
+  constexpr int STAGES = 3;
+  using Pipe = DmaPipe<TS, 2, 3, STAGES>;
+  using SM = typename Pipe::SM;
+  const HiddenParams& p = pp.h;
+  int bx, by, z;
+  if (!pp.map.locate(blockIdx.x, bx, by, z)) return;
+  const int m0 = bx * TS::BM, n0 = by * TS::BN;
+  const int nk = p.d / DMA_BK;
+  const int halves = min(TS::BN, p.dh - n0) / 64;          // valid 64-column halves of this tile
+  DmaPhase<2> ph[3];
+  // the one-accumulator phase first: the two-accumulator K-steps in front of the input stages are the longer ones,
+  // which gives the input copies more time to land
+  ph[0].a = token_operand<TS>(p.Y, p.bsy, p.ldy, z, m0, p.T);
+  ph[0].b[0] = weight_operand_ks(p.G1, p.bsw, p.dh, z, n0, p.dh);
+  ph[0].b[1] = ph[0].b[0];
+  ph[0].nb = 1;
+  ph[0].K = p.d;
+  ph[1].a = token_operand<TS>(p.X, p.bsx, p.ldx, z, m0, p.T);
+  ph[1].b[0] = weight_operand(p.G0, p.bsw, p.d, z, n0, p.dh);
+  ph[1].b[1] = weight_operand(p.G2, p.bsw, p.d, z, n0, p.dh);
+  ph[1].nb = 2;
+  ph[1].K = p.d;
+  ph[2].a = token_operand<TS>(reinterpret_cast<const uint16_t*>(p.I0) + n0, p.bsi, p.dh, z, m0, p.T);
+  ph[2].b[0] = token_operand<TS>(reinterpret_cast<const uint16_t*>(p.I1) + n0, p.bsi, p.dh, z, m0, p.T);
+  ph[2].b[1] = token_operand<TS>(reinterpret_cast<const uint16_t*>(p.I2) + n0, p.bsi, p.dh, z, m0, p.T);
+  ph[2].nb = 2;
+  ph[2].K = halves * 64;
+  f32x16 ag[2][TS::TM][TS::TN], ay[1][TS::TM][TS::TN];
+  zero_acc<TS>(ag[0]);
+  zero_acc<TS>(ag[1]);
+  zero_acc<TS>(ay[0]);
+  LACT_TS(0);
+  Pipe pipe(smem, ph);
+  const bool loader = Pipe::is_loader();
+  if (loader) {
+    pipe.template load_all<Pipe::loads(1)>();
+  } else {
+    int step = 0;
+    pipe.template run_phase<1, false, true>(nk, step, ay);
+    pipe.template run_phase<2>(nk, step, ag);
+    LACT_TS(1);
+    for (int i = 0; i < halves; ++i) __syncthreads();   // the input stages land behind these barriers
+  }
+  LACT_TS(2);
+  // input half h sits in the stage of K-step 2 nk + h
+  if (!loader) {
+    // the products enter the pointwise part as bf16 values: packing them in pairs first halves the registers
+    // the accumulators hold while that part runs
+    uint32_t pz[3][TS::TM][TS::TN][8];
+#pragma unroll
+    for (int tm = 0; tm < TS::TM; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < TS::TN; ++tn)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          pz[0][tm][tn][e] = (uint32_t)f32_to_bf16(ag[0][tm][tn][2 * e]) | ((uint32_t)f32_to_bf16(ag[0][tm][tn][2 * e + 1]) << 16);
+          pz[1][tm][tn][e] = (uint32_t)f32_to_bf16(ay[0][tm][tn][2 * e]) | ((uint32_t)f32_to_bf16(ay[0][tm][tn][2 * e + 1]) << 16);
+          pz[2][tm][tn][e] = (uint32_t)f32_to_bf16(ag[1][tm][tn][2 * e]) | ((uint32_t)f32_to_bf16(ag[1][tm][tn][2 * e + 1]) << 16);
+          // opaque to the optimiser: otherwise it undoes the packing and keeps every product as a float of its own
+          asm volatile("" : "+v"(pz[0][tm][tn][e]), "+v"(pz[1][tm][tn][e]), "+v"(pz[2][tm][tn][e]));
+        }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int half = wave % TS::WAVES_N;
+    char* st = smem + ((2 * nk + half) % STAGES) * SM::STAGE;
+    const int row_l = (wave / TS::WAVES_N) * TS::WM + (lane & 31);
+    const uint32_t key = (uint32_t)((lane >> 1) & 7) << 4;
+    char* lb = st + row_l * 128 + ((lane >> 5) << 3);
+#pragma unroll
+    for (int tm = 0; tm < TS::TM; ++tm) {
+      const int ml = quad_m<TS>(tm), m = m0 + ml;
+      const bool mv = m < p.T;
+      const float l0 = mv ? p.lr0[z * p.bslr + m] : 0.f, l1 = mv ? p.lr1[z * p.bslr + m] : 0.f;
+      const float l2 = mv ? p.lr2[z * p.bslr + m] : 0.f;
+      float s0 = 0.f, s1 = 0.f, s2 = 0.f;
+#pragma unroll
+      for (int tn = 0; tn < TS::TN; ++tn)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int nl = quad_n<TS>(tn, g);
+          const bool nv = n0 + nl < p.dh;
+          char* q0 = lb + tm * 32 * 128 + (((uint32_t)(tn * 4 + g) << 4) ^ key);
+          float i0[4], i1[4], i2[4], o0[4], o1[4], o2[4];
+          Elem<uint16_t>::load4(reinterpret_cast<const uint16_t*>(q0), i0);
+          Elem<uint16_t>::load4(reinterpret_cast<const uint16_t*>(q0 + SM::A_BYTES), i1);
+          Elem<uint16_t>::load4(reinterpret_cast<const uint16_t*>(q0 + SM::A_BYTES + SM::B_BYTES), i2);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float gg = i0[j], h2 = i1[j], dh = i2[j];
+            const uint32_t w0_ = pz[0][tm][tn][2 * g + (j >> 1)], w1_ = pz[1][tm][tn][2 * g + (j >> 1)], w2_ = pz[2][tm][tn][2 * g + (j >> 1)];
+            const float gz0 = __uint_as_float((j & 1) ? (w0_ & 0xffff0000u) : (w0_ << 16));
+            const float gz1 = __uint_as_float((j & 1) ? (w1_ & 0xffff0000u) : (w1_ << 16));
+            const float gz2 = __uint_as_float((j & 1) ? (w2_ & 0xffff0000u) : (w2_ << 16));
+            const SiluParts s = silu_parts(gg);
+            const UpdatePointwise u = update_pointwise<uint16_t>(gg, h2, dh, s);
+            if (mv && nv) { s0 += gz0 * u.dgpre; s1 += gz1 * u.hid; s2 += gz2 * u.dh2; }
+            const float ghid = gz1 * l1, gdh2 = gz2 * l2, gdg = gz0 * l0;
+            o0[j] = ghid * h2 * s.d1 + gdh2 * dh * s.d1 + gdg * dh * h2 * s.d2;
+            o1[j] = gdh2 * s.silu + gdg * h2 * s.d1;
+            o2[j] = ghid * s.silu + gdg * dh * s.d1;
+          }
+          Elem<uint16_t>::store4(reinterpret_cast<uint16_t*>(q0), o0[0], o0[1], o0[2], o0[3]);
+          Elem<uint16_t>::store4(reinterpret_cast<uint16_t*>(q0 + SM::A_BYTES), o1[0], o1[1], o1[2], o1[3]);
+          Elem<uint16_t>::store4(reinterpret_cast<uint16_t*>(q0 + SM::A_BYTES + SM::B_BYTES), o2[0], o2[1], o2[2], o2[3]);
+        }
+      store_row_partials<TS>(p, 0, tm, m, z, s0, by);
+      store_row_partials<TS>(p, 1, tm, m, z, s1, by);
+      store_row_partials<TS>(p, 2, tm, m, z, s2, by);
+    }
+  }
+  __syncthreads();
+  LACT_TS(3);
+  // copy the result stages out: 8 granules of 16 bytes per row and half, rows of 128 bytes stay whole
+  {
+    uint16_t* outs[3] = {reinterpret_cast<uint16_t*>(p.O0), reinterpret_cast<uint16_t*>(p.O1), reinterpret_cast<uint16_t*>(p.O2)};
+    const size_t off = z * p.bso + (size_t)m0 * p.dh + n0;
+    const int rows = min(TS::BM, p.T - m0);
+    for (int id = threadIdx.x; id < halves * TS::BM * 8; id += DMA_THREADS) {
+      const int j = id & 7, r = (id >> 3) % TS::BM, h = id / (8 * TS::BM);
+      if (r >= rows) continue;
+      const char* src = smem + ((2 * nk + h) % STAGES) * SM::STAGE + r * 128 + ((j ^ ((r >> 1) & 7)) << 4);
+      const size_t o = off + (size_t)r * p.dh + h * 64 + j * 8;
+      *reinterpret_cast<uint4*>(outs[0] + o) = *reinterpret_cast<const uint4*>(src);
+      *reinterpret_cast<uint4*>(outs[1] + o) = *reinterpret_cast<const uint4*>(src + SM::A_BYTES);
+      *reinterpret_cast<uint4*>(outs[2] + o) = *reinterpret_cast<const uint4*>(src + SM::A_BYTES + SM::B_BYTES);
+    }
+  }
+  LACT_TS(4);
 }
 
 // ------------------------------------------------------------------------------------------------

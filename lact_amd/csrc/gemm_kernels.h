@@ -116,6 +116,8 @@ struct HiddenParams {
   const void* G0; const void* G1; const void* G2;
   void* O0; void* O1; void* O2; void* O3; void* O4; void* O5;  // [b, T, dh] outputs, type T
   long long bso;
+  // update backward from kept pre-activations: I0 = k W0^T, I1 = k W2^T, I2 = v W1 as the forward rounded them
+  const void* I0; const void* I1; const void* I2; long long bsi;
   float* lrpart; long long lrpart_stride;  // partial row sums: [3][nparts][b*Tcap]; stride between parts
   long long lrpart_mat_stride;
   int Tcap;

@@ -200,6 +200,12 @@ struct Plan {
   size_t mat3 = 0;  // 3*b*elems
   // saved
   size_t s_n0, s_wf, s_wc, s_main, s_d, s_mbar, s_u, s_g16, s_norms, s_xb, s_ab, s_bb, saved_bytes;
+  // Kept for the backward on the asynchronous-copy path: per update, six token-major arrays [b][T][dh] -- the three
+  // lr-scaled operands of the fast-weight gradient GEMMs and the three rounded pre-activations they came from.
+  // 288 GB of HBM make keeping them cheaper than the three GEMMs that would recompute them.
+  bool keep_pre = false;
+  std::vector<size_t> s_pre;   // by update index
+  std::vector<int> pre_T;
   // scratch
   size_t t_h[6], t_partial, t_lrpart, t_xf[2], t_xbtmp, t_ss, t_dot, t_mdot, t_gwhat[2], t_gwcur, t_gmcarry, t_gc,
       t_gxf[2], t_gxb[2], t_sg, t_gas, t_gn0, t_hs[3], t_partial_side, t_gwside[2], t_nssync, scratch_bytes;
@@ -283,6 +289,14 @@ struct Plan {
     const size_t sq3 = sq_total;
     s_ab = muon ? sv.take((size_t)nupd * std::max(1, S) * sq3 * nsz) : 0;
     s_bb = muon ? sv.take((size_t)nupd * std::max(1, S) * sq3 * nsz) : 0;
+    keep_pre = bf16 && d.d % 64 == 0 && d.dh % 64 == 0;
+    s_pre.clear(); pre_T.clear();
+    if (keep_pre)
+      for (const auto& st : steps)
+        if (st.kind == LACT_UPDATE) {
+          pre_T.push_back(st.end - st.start);
+          s_pre.push_back(sv.take((size_t)6 * d.b * (st.end - st.start) * d.dh * esz));
+        }
     saved_bytes = sv.off + 256;
 
     Bump sc;
@@ -516,12 +530,23 @@ struct Runner {
   TN* ab(int u, int it) const { return reinterpret_cast<TN*>(sv + P.s_ab) + ((size_t)u * std::max(1, P.S) + it) * sq3(); }
   TN* bb(int u, int it) const { return reinterpret_cast<TN*>(sv + P.s_bb) + ((size_t)u * std::max(1, P.S) + it) * sq3(); }
   T* h(int i) const { return reinterpret_cast<T*>(sc + hsel[i]); }
+  // kept array i (0..2: lr-scaled operands, 3..5: pre-activations) of update u; batch stride pre_bs(u)
+  T* pre(int u, int i) const { return reinterpret_cast<T*>(sv + P.s_pre[u]) + (size_t)i * d.b * P.pre_T[u] * d.dh; }
+  long long pre_bs(int u) const { return (long long)P.pre_T[u] * d.dh; }
   static constexpr bool kBf16 = std::is_same<T, uint16_t>::value;
   static constexpr bool kNsBf16 = std::is_same<TN, uint16_t>::value;
 
+  // the hidden-stage kernels with asynchronous copies need bf16 and whole 64-element K-steps
+  bool dma_hidden() const { return kBf16 && d.d % 64 == 0; }
+  // row-partial slots the update-backward hidden kernel in use writes: (hidden tiles) x (wave columns)
+  int lr_parts() const {
+    if (!dma_hidden()) return ceil_div(d.dh, TSB::BN) * TSB::WAVES_N;
+    if (P.keep_pre) return ceil_div(d.dh, TS_SQ::BN) * TS_SQ::WAVES_N;
+    return ceil_div(d.dh, TS_BWD::BN) * TS_BWD::WAVES_N;
+  }
   void launch_hidden(int which, const HiddenParams& hp, int ver, int T_) const {
     const double f = (double)T_ * d.d * d.dh * d.b;
-    if (kBf16 && d.d % 64 == 0) {
+    if (dma_hidden()) {
       if constexpr (kBf16) {
       HiddenDmaParams q;
       q.h = hp;
@@ -536,10 +561,12 @@ struct Runner {
       LACT_BIG_LDS(k_update_hidden_dma<TS_SQ>, SM3);
       LACT_BIG_LDS(k_apply_bwd_hidden_dma<TS_SQ>, SM3);
       LACT_BIG_LDS(k_update_bwd_hidden_dma<TS_BWD>, SM6);
+      LACT_BIG_LDS(k_update_bwd_hidden_kept_dma<TS_SQ>, SM3);
       if (which == 0) LACT_LAUNCH_SMEM("k_apply_hidden_dma", "apply_hidden", 4.0 * f, (k_apply_hidden_dma<TS_SQ>), g3, dim3(DMA_THREADS), SM3, s, q);
       if (which == 1) LACT_LAUNCH_SMEM("k_update_hidden_dma", "update_hidden", 6.0 * f, (k_update_hidden_dma<TS_SQ>), g3, dim3(DMA_THREADS), SM3, s, q);
       if (which == 2) LACT_LAUNCH_SMEM("k_apply_bwd_hidden_dma", "apply_bwd_hidden", 6.0 * f, (k_apply_bwd_hidden_dma<TS_SQ>), g3, dim3(DMA_THREADS), SM3, s, q);
       if (which == 3) LACT_LAUNCH_SMEM("k_update_bwd_hidden_dma", "update_bwd_hidden", 12.0 * f, (k_update_bwd_hidden_dma<TS_BWD>), g6, dim3(DMA_THREADS), SM6, s, q);
+      if (which == 4) LACT_LAUNCH_SMEM("k_update_bwd_hidden_kept_dma", "update_bwd_hidden", 6.0 * f, (k_update_bwd_hidden_kept_dma<TS_SQ>), g3, dim3(DMA_THREADS), SM3, s, q);
       }
     } else {
       dim3 ga(ceil_div(T_, TSA::BM), ceil_div(d.dh, TSA::BN), d.b), gb(ceil_div(T_, TSB::BM), ceil_div(d.dh, TSB::BN), d.b);
@@ -654,6 +681,8 @@ struct Runner {
       LACT_LAUNCH("k_init_state", "k_init_state", 0.0, (k_init_state<T>), rowgrid, dim3(256), s, p);
     }
     int ver = 0, u = 0;
+    T* upd_z[3] = {nullptr, nullptr, nullptr};   // lr-scaled operands of the current update's gradient GEMMs
+    long long upd_zbs = 0;
     bool side_used = false;
     // Apply steps only need their weight version, which is final once they are met in program order.  They are
     // held back and enqueued on the side stream at the point of the following update where the chip is least
@@ -695,8 +724,16 @@ struct Runner {
       {
         HiddenParams hp = hidden_params(T_, kc, d.k_ld, d.k_bs, vc, d.v_ld, d.v_bs, ver);
         hp.lr0 = lr0 + st.start; hp.lr1 = lr1 + st.start; hp.lr2 = lr2 + st.start; hp.bslr = d.kv_len;
-        hp.O0 = h(0); hp.O1 = h(1); hp.O2 = h(2);
+        T* z0 = h(0); T* z1 = h(1); T* z2 = h(2);
+        long long zbs = hbs();
+        if (P.keep_pre) {
+          z0 = pre(u, 0); z1 = pre(u, 1); z2 = pre(u, 2); zbs = pre_bs(u);
+          hp.O3 = pre(u, 3); hp.O4 = pre(u, 4); hp.O5 = pre(u, 5);
+          hp.bso = zbs;
+        }
+        hp.O0 = z0; hp.O1 = z1; hp.O2 = z2;
         launch_hidden(1, hp, ver, T_);
+        upd_z[0] = z0; upd_z[1] = z1; upd_z[2] = z2; upd_zbs = zbs;
       }
       int dw_slots = 0;
       {
@@ -704,11 +741,11 @@ struct Runner {
         memset(jobs, 0, sizeof(jobs));
         jobs[0].nterms = jobs[1].nterms = jobs[2].nterms = 1;
         jobs[0].M = d.dh; jobs[0].N = d.d;
-        set_tr_term(jobs[0].t[0], h(0), d.dh, hbs(), kc, d.k_ld, d.k_bs);
+        set_tr_term(jobs[0].t[0], upd_z[0], d.dh, upd_zbs, kc, d.k_ld, d.k_bs);
         jobs[1].M = d.d; jobs[1].N = d.dh;
-        set_tr_term(jobs[1].t[0], vc, d.v_ld, d.v_bs, h(1), d.dh, hbs());
+        set_tr_term(jobs[1].t[0], vc, d.v_ld, d.v_bs, upd_z[1], d.dh, upd_zbs);
         jobs[2].M = d.dh; jobs[2].N = d.d;
-        set_tr_term(jobs[2].t[0], h(2), d.dh, hbs(), kc, d.k_ld, d.k_bs);
+        set_tr_term(jobs[2].t[0], upd_z[2], d.dh, upd_zbs, kc, d.k_ld, d.k_bs);
         dw_slots = token_reduce("update_dw", jobs, T_);
       }
       // the first update has no earlier momentum state to weigh: its mean is never used
@@ -1110,6 +1147,9 @@ struct Runner {
       const T* vc = v + (size_t)st.start * d.v_ld;
       T* gcm = scr<T>(P.t_gc);
       T* g0 = gcm; T* g1 = gcm + (size_t)d.b * P.g.elems; T* g2 = gcm + (size_t)2 * d.b * P.g.elems;
+      // lr-scaled operands of the forward's gradient GEMMs: kept by the forward, or written again by the hidden kernel
+      T* z0 = h(3); T* z1 = h(4); T* z2 = h(5);
+      long long zbs = hbs();
       {
         HiddenParams hp = hidden_params(T_, kc, d.k_ld, d.k_bs, vc, d.v_ld, d.v_bs, vprev);
         hp.lr0 = lr0 + st.start; hp.lr1 = lr1 + st.start; hp.lr2 = lr2 + st.start; hp.bslr = d.kv_len;
@@ -1118,9 +1158,14 @@ struct Runner {
         hp.lrpart = scr<float>(P.t_lrpart);
         hp.lrpart_stride = (long long)d.b * P.Tcap;
         hp.lrpart_mat_stride = (long long)P.lr_slots * d.b * P.Tcap;
+        if (P.keep_pre) {
+          hp.I0 = pre(u, 3); hp.I1 = pre(u, 4); hp.I2 = pre(u, 5); hp.bsi = pre_bs(u);
+          hp.O3 = hp.O4 = hp.O5 = nullptr;
+          z0 = pre(u, 0); z1 = pre(u, 1); z2 = pre(u, 2); zbs = pre_bs(u);
+        }
         wait_main_dq();
         wait_tail();
-        launch_hidden(3, hp, vprev, T_);
+        launch_hidden(P.keep_pre ? 4 : 3, hp, vprev, T_);
       }
       const bool acc_kv = seen_kv.accumulate(st.start, st.end);
       // worth a hand-over only when an earlier update's chain follows on the caller's stream
@@ -1131,8 +1176,8 @@ struct Runner {
       }
       {  // dk = (dgate*lr0) G0 + (dh2*lr2) G2 + gG W0 + gH2 W2
         auto p = row_params<4>();
-        set_term(p.t[0], h(3), d.dh, hbs(), g0, d.d, P.g.elems, d.dh);
-        set_term(p.t[1], h(5), d.dh, hbs(), g2, d.d, P.g.elems, d.dh);
+        set_term(p.t[0], z0, d.dh, zbs, g0, d.d, P.g.elems, d.dh);
+        set_term(p.t[1], z2, d.dh, zbs, g2, d.d, P.g.elems, d.dh);
         set_term(p.t[2], h(0), d.dh, hbs(), wc(vprev, 0), d.d, P.g.elems, d.dh);
         set_term(p.t[3], h(2), d.dh, hbs(), wc(vprev, 2), d.d, P.g.elems, d.dh);
         p.M = T_; p.N = d.d; p.out = dk + (size_t)st.start * d.d; p.ldo = d.d; p.bso = (long long)d.kv_len * d.d;
@@ -1141,7 +1186,7 @@ struct Runner {
       }
       {  // dv = (hidden*lr1) G1^T + gDH W1^T
         auto p = row_params<2>();
-        set_term(p.t[0], h(4), d.dh, hbs(), g1, d.dh, P.g.elems, d.dh);
+        set_term(p.t[0], z1, d.dh, zbs, g1, d.dh, P.g.elems, d.dh);
         set_term(p.t[1], h(1), d.dh, hbs(), wc(vprev, 1), d.dh, P.g.elems, d.dh);
         p.M = T_; p.N = d.d; p.out = dv + (size_t)st.start * d.d; p.ldo = d.d; p.bso = (long long)d.kv_len * d.d;
         p.accumulate = acc_kv;
@@ -1149,7 +1194,7 @@ struct Runner {
       }
       LACT_LAUNCH("k_lr_reduce", "k_lr_reduce", 0.0, k_lr_reduce, dim3(ceil_div(T_, 256), d.b, 3), dim3(256), s, scr<float>(P.t_lrpart),
                          (long long)P.lr_slots * d.b * P.Tcap, (long long)d.b * P.Tcap,
-                  kBf16 ? ceil_div(d.dh, TS_BWD::BN) * TS_BWD::WAVES_N : ceil_div(d.dh, TSB::BN) * TSB::WAVES_N, P.Tcap, dlr0, dlr1, dlr2,
+                  lr_parts(), P.Tcap, dlr0, dlr1, dlr2,
                          (long long)d.kv_len, st.start, T_);
       if (use_tail) {
         s = s_main;
