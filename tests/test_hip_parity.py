@@ -148,20 +148,30 @@ def block_causal_pair(C, use_muon, prenorm=False):
 @pytest.mark.parametrize("b,L,d,dh,C,mom,prenorm", [
     (2, 3 * 64 + 5, 64, 64, 64, False, False), (2, 3 * 64 + 5, 64, 64, 64, True, False),
     (2, 2 * 96 + 17, 64, 128, 96, True, False), (2, 2 * 96 + 17, 128, 64, 96, True, True),
-    (3, 4 * 200, 384, 384, 200, True, False), (1, 100, 64, 64, 128, True, False)])
+    (3, 4 * 200, 384, 384, 200, True, False), (1, 100, 64, 64, 128, True, False),
+    (2, 2 * 96 + 17, 40, 136, 96, True, False),    # d not a multiple of 64: generic tile kernels, two hidden tiles
+    (2, 2 * 96 + 17, 64, 192, 96, True, False)])   # dh = 128 + 64: a half-valid hidden tile on the asynchronous-copy path
 def test_block_causal_bf16_no_muon(b, L, d, dh, C, mom, prenorm):
     say("block_causal bf16 no muon", b, L, d, dh, C, mom, prenorm)
     inp = problem(b, L, d, dh, 7, torch.bfloat16, momentum=mom)
-    res, ref = run_both(*block_causal_pair(C, False, prenorm), inp, AC)
+    res, ref, r64 = run_both(*block_causal_pair(C, False, prenorm), inp, AC, ref64=True)
     errs = compare(res, ref)
     say("  ", errs)
     assert res["out"].dtype == torch.bfloat16
-    assert max(errs.values()) < 1e-2                       # north-star bf16 bound
+    # d loss / d momentum is one dot product <g, M_prev> per head and chunk: with few, short rows the bf16 oracle
+    # itself sits percent away from exact arithmetic there, so that entry is held to the oracle's own distance
+    floor = O.rel_l2(ref["momentum"], r64["momentum"]) if "momentum" in errs else 0.0
+    for n, e in errs.items():
+        if n == "momentum" and floor > 5e-3:
+            say("   momentum: oracle-vs-f64", floor, "hip-vs-f64", O.rel_l2(res[n], r64[n]))
+            assert O.rel_l2(res[n], r64[n]) <= 1.5 * floor + 2e-3
+        else:
+            assert e < 1e-2, n                             # north-star bf16 bound
 
 
 @pytest.mark.parametrize("b,L,d,dh,C,mom,prenorm", [
     (2, 3 * 64 + 5, 64, 64, 64, True, False), (2, 2 * 96 + 17, 64, 128, 96, True, True),
-    (2, 2 * 96 + 17, 128, 64, 96, False, False)])
+    (2, 2 * 96 + 17, 128, 64, 96, False, False), (2, 2 * 96 + 17, 40, 136, 96, True, False)])
 def test_block_causal_fp32_no_muon(b, L, d, dh, C, mom, prenorm):
     say("block_causal fp32 no muon", b, L, d, dh, C, mom, prenorm)
     inp = problem(b, L, d, dh, 8, torch.float32, momentum=mom)
