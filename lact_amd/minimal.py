@@ -30,7 +30,7 @@ def bidirectional_lact_swiglu(w0, w1, w2, q, k, v, lr0, lr1, lr2, use_muon: bool
     """bidirectional_lact_layer.py:74-160: one update on every token, then apply to every query.
     muon_mode="reference" reproduces :139-146 (the orthogonalised gradient replaces the weight and the
     raw gradient is added); "intended" adds the orthogonalised gradient to the weight."""
-    prog = Program(steps=((LACT_UPDATE, 0, k.shape[1], 0), (LACT_APPLY, 0, q.shape[1], 0)), out_len=q.shape[1],
+    prog = Program(steps=((LACT_UPDATE, 0, k.shape[1], 0), (LACT_APPLY, 0, q.shape[1], 0)), out_len=q.shape[1], return_state=False,
                    ns_coeffs=NS5_COEFFS if use_muon else None,
                    muon_replaces_weight=(use_muon and muon_mode == "reference"),
                    ns_mode=ops._ns_mode(q))

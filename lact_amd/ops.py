@@ -42,6 +42,9 @@ class Program:
     # gradient cat(dw0, dw2); eps inside the sqrt of the row renorm
     muon_stacked: bool = False
     renorm_eps_in_sqrt: bool = False
+    # callers that only use the output (the block-causal and bidirectional functions) spare the copies of the final
+    # fast weights and momentum states: run_program then returns None in their places
+    return_state: bool = True
 
     @property
     def n_updates(self) -> int:
@@ -163,8 +166,8 @@ class _LactProgramFn(torch.autograd.Function):
         saved_bytes, scratch_bytes = call.sizes()
         saved = torch.empty(saved_bytes, dtype=torch.uint8, device=q.device)
         scratch = torch.empty(scratch_bytes, dtype=torch.uint8, device=q.device)
-        w_out = [torch.empty_like(w) for w in wf]
-        m_out = [torch.empty_like(w) for w in wf] if mom is not None else [None, None, None]
+        w_out = [torch.empty_like(w) for w in wf] if prog.return_state else [None, None, None]
+        m_out = [torch.empty_like(w) for w in wf] if (mom is not None and prog.return_state) else [None, None, None]
         stream = ctypes.c_void_p(torch.cuda.current_stream(q.device).cuda_stream)
         with torch.cuda.device(q.device):
             _lib.check(L.lact_forward(ctypes.byref(call.desc), _ptr(wf[0]), _ptr(wf[1]), _ptr(wf[2]), _ptr(qa), _ptr(ka),
@@ -183,6 +186,8 @@ class _LactProgramFn(torch.autograd.Function):
         if v is not None and v.dtype == torch.float32 and act == torch.bfloat16:
             out_dtype = torch.float32          # zeros_like(v) receives the bf16 products
         res_out = out if out.dtype == out_dtype else out.to(out_dtype)
+        if not prog.return_state:
+            return (res_out, None, None, None, None, None, None)
         m_ret = tuple(m if m is not None else torch.zeros_like(wf[i]) for i, m in enumerate(m_out))
         return (res_out, w_out[0], w_out[1], w_out[2]) + m_ret
 

@@ -28,7 +28,7 @@ def zeropower_via_newtonschulz5(G: torch.Tensor) -> torch.Tensor:
 
 def _block_causal(w0, w1, w2, q, k, v, lr0, lr1, lr2, chunk_size, use_muon, momentum, prenorm,
                   muon_stacked=False, renorm_eps_in_sqrt=False):
-    prog = Program(steps=block_causal_steps(k.shape[1], chunk_size), out_len=q.shape[1],
+    prog = Program(steps=block_causal_steps(k.shape[1], chunk_size), out_len=q.shape[1], return_state=False,
                    ns_coeffs=NS5_COEFFS if use_muon else None, prenorm=prenorm,
                    ns_mode=ops._ns_mode(q), muon_stacked=muon_stacked and use_muon,
                    renorm_eps_in_sqrt=renorm_eps_in_sqrt)
