@@ -67,6 +67,9 @@ typedef struct lact_desc {
   /* The two places where the fused-kernel driver differs in semantics (ttt_operation_fused_kernel.py): */
   int32_t muon_stacked;          /* Newton-Schulz on cat(dw0, dw2) [2dh, d] and on dw1 (:168-170, :308-310) */
   int32_t renorm_eps_in_sqrt;    /* y = w / sqrt(|w|^2 + eps) * n0 (:172-173; l2norm_triton_kernels.py:205-214) */
+  /* No lact_backward call follows (inference, torch.no_grad): the forward keeps no activations for it, `saved` is
+   * smaller, and lact_backward refuses the descriptor.  No counterpart in the reference, where autograd decides. */
+  int32_t forward_only;
 } lact_desc_t;
 
 const char* lact_last_error(void);

@@ -29,7 +29,7 @@ class Desc(Structure):
         ("detach_norms", c_int32), ("muon_replaces_weight", c_int32), ("ns_mode", c_int32),
         ("q_bs", c_int64), ("k_bs", c_int64), ("v_bs", c_int64), ("o_bs", c_int64), ("do_bs", c_int64),
         ("q_ld", c_int32), ("k_ld", c_int32), ("v_ld", c_int32), ("o_ld", c_int32), ("do_ld", c_int32),
-        ("muon_stacked", c_int32), ("renorm_eps_in_sqrt", c_int32),
+        ("muon_stacked", c_int32), ("renorm_eps_in_sqrt", c_int32), ("forward_only", c_int32),
     ]
 
 

@@ -289,7 +289,7 @@ struct Plan {
     const size_t sq3 = sq_total;
     s_ab = muon ? sv.take((size_t)nupd * std::max(1, S) * sq3 * nsz) : 0;
     s_bb = muon ? sv.take((size_t)nupd * std::max(1, S) * sq3 * nsz) : 0;
-    keep_pre = bf16 && d.d % 64 == 0 && d.dh % 64 == 0;
+    keep_pre = bf16 && d.d % 64 == 0 && d.dh % 64 == 0 && !d.forward_only;
     s_pre.clear(); pre_T.clear();
     if (keep_pre)
       for (const auto& st : steps)
@@ -1513,6 +1513,7 @@ int lact_backward(const lact_desc_t* desc, const void* q, const void* k, const v
                   float* dlr2, float* dmomentum, void* stream) {
   Plan P;
   if (P.build(desc)) return -1;
+  if (P.d.forward_only) return fail("the forward ran with forward_only set: nothing was kept for a backward pass");
   if (check_ptrs({q, dout, saved, scratch, dw0, dw1, dw2, dq}, "backward tensors")) return -1;
   if (P.nupd > 0 && check_ptrs({k, v, lr0, lr1, lr2, dk, dv, dlr0, dlr1, dlr2}, "k, v, lr and their gradients")) return -1;
   if (P.nupd > 0 && P.momentum && (!momentum || !dmomentum)) return fail("use_momentum set but momentum or dmomentum is null");

@@ -163,6 +163,7 @@ class _LactProgramFn(torch.autograd.Function):
         out = alloc((b, prog.out_len, d), dtype=act, device=q.device)
         call = _Call(prog, b, d, dh, qa, ka, va, out)
         call.desc.use_momentum = int(mom is not None)
+        call.desc.forward_only = int(not any(ctx.needs_input_grad))
         saved_bytes, scratch_bytes = call.sizes()
         saved = torch.empty(saved_bytes, dtype=torch.uint8, device=q.device)
         scratch = torch.empty(scratch_bytes, dtype=torch.uint8, device=q.device)
