@@ -38,12 +38,12 @@ CONFIGS = {
 # HBM bytes per launch at config 1 (read + write), from the FETCH_SIZE / WRITE_SIZE counters of two
 # `rocprofv3 --pmc` runs scaled by a 1 GiB copy (profiles/c1_fwd_bwd_hbm_traffic_pmc.txt); MiB.
 MEASURED_TRAFFIC_MIB = {
-    "k_ns_fused<192x192,bwd>": 730.5 + 347.6,
+    "k_ns_fused<192x192,bwd>": 730.8 + 347.6,
     "k_ns_fused<192x192,fwd>": 424.2 + 346.4,
     "k_token_reduce_dma<192x192>": 127.0 + 27.0,
-    "k_update_bwd_hidden_dma": 128.7 + 148.5,
+    "k_update_bwd_hidden_kept_dma": 151.3 + 74.2,
     "k_apply_bwd_hidden_dma": 78.1 + 72.0,
-    "k_update_hidden_dma": 77.9 + 72.0,
+    "k_update_hidden_dma": 79.0 + 144.0,
     "k_apply_hidden_dma": 33.3 + 24.0,
 }
 
