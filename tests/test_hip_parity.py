@@ -471,6 +471,74 @@ def test_config4_full_size_properties():
     full_size_properties(12, 32760, 128, 256, 4680, 1004, False)
 
 
+def test_calls_on_two_caller_streams():
+    """Two independent problems enqueued on two caller streams at once (forward and backward each), as a caller with
+    its own stream pool would: the library's side streams, the ordering of the fused Newton-Schulz kernels across
+    streams and the shared event pool must not mix them up.  Same bits as the same calls on one stream."""
+    say("two caller streams")
+    b, L, d, dh, C = 2, 3 * 384, 384, 384, 384
+    inps = [problem(b, L, d, dh, seed=91 + i, act=torch.bfloat16) for i in range(2)]
+    gos = [torch.randn(b, L, d, generator=torch.Generator().manual_seed(7 + i)).bfloat16().to(DEV) for i in range(2)]
+
+    def run(streams):
+        ts = [clone_to(inp, DEV) for inp in inps]
+        torch.cuda.synchronize()
+        outs, grads = [None, None], [None, None]
+        for rep in range(2):
+            for i in range(2):
+                with torch.cuda.stream(streams[i]):
+                    outs[i] = T.block_causal_lact_swiglu(*args9(ts[i]), C, True, ts[i]["momentum"])
+            for i in range(2):
+                with torch.cuda.stream(streams[i]):
+                    grads[i] = grads_of(outs[i], ts[i], gos[i])
+        torch.cuda.synchronize()
+        return outs, grads
+    cur = torch.cuda.current_stream()
+    o1, g1 = run([cur, cur])
+    o2, g2 = run([torch.cuda.Stream(), torch.cuda.Stream()])
+    for i in range(2):
+        assert torch.equal(o1[i], o2[i])
+        for n in g1[i]:
+            assert torch.equal(g1[i][n], g2[i][n]), n
+
+
+def test_calls_from_two_host_threads():
+    """Two host threads, each with a stream of its own, run forward + backward of different problems at the same
+    time (the enqueue of a program is serialised inside the library; execution is not).  Same bits as one thread."""
+    say("two host threads")
+    import threading
+    b, L, d, dh, C = 2, 3 * 256, 128, 256, 256
+    inps = [problem(b, L, d, dh, seed=191 + i, act=torch.bfloat16) for i in range(2)]
+    gos = [torch.randn(b, L, d, generator=torch.Generator().manual_seed(17 + i)).bfloat16().to(DEV) for i in range(2)]
+
+    def one(i, stream, res):
+        try:
+            with torch.cuda.stream(stream):
+                for _ in range(3):
+                    t = clone_to(inps[i], DEV)
+                    out = T.block_causal_lact_swiglu(*args9(t), C, True, t["momentum"])
+                    res[i] = (out, grads_of(out, t, gos[i]))
+            stream.synchronize()
+        except Exception as e:   # surfaces in the main thread below
+            res[i] = e
+    ref = [None, None]
+    for i in range(2):
+        one(i, torch.cuda.current_stream(), ref)
+    torch.cuda.synchronize()
+    res = [None, None]
+    th = [threading.Thread(target=one, args=(i, torch.cuda.Stream(), res)) for i in range(2)]
+    for t_ in th:
+        t_.start()
+    for t_ in th:
+        t_.join()
+    torch.cuda.synchronize()
+    for i in range(2):
+        assert not isinstance(res[i], Exception), res[i]
+        assert torch.equal(res[i][0], ref[i][0])
+        for n in ref[i][1]:
+            assert torch.equal(res[i][1][n], ref[i][1][n]), n
+
+
 @pytest.mark.parametrize("prenorm", [False, True])
 def test_stream_overlap_is_bit_identical(prenorm):
     """The apply steps run on the library's second stream beside the update chain (forked and joined with
