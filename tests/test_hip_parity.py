@@ -471,6 +471,47 @@ def test_config4_full_size_properties():
     full_size_properties(12, 32760, 128, 256, 4680, 1004, False)
 
 
+def test_graph_capture_replays_match_eager():
+    """Forward + backward captured into a HIP graph (the library forks and joins its side streams with events
+    only, and clears memory with kernels): three replays on fresh inputs, with eager work and synchronisations in
+    between, each bit-identical to the eager call on the same inputs."""
+    say("graph capture")
+    b, L, d, dh, C = 2, 3 * 384, 384, 384, 384
+    inp = problem(b, L, d, dh, seed=55, act=torch.bfloat16)
+    st = clone_to(inp, DEV)
+    go = torch.randn(b, L, d, generator=torch.Generator().manual_seed(9)).bfloat16().to(DEV)
+
+    def run():
+        out = T.block_causal_lact_swiglu(*args9(st), C, True, st["momentum"])
+        return out, grads_of(out, st, go)
+    run()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):               # warm-up on a side stream, as torch asks before a capture
+        run()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_g, grads_g = run()
+    torch.cuda.synchronize()
+    gen = torch.Generator().manual_seed(123)
+    for rep in range(3):
+        with torch.no_grad():
+            st["q"].copy_(torch.nn.functional.normalize(torch.randn(b, L, d, generator=gen), dim=-1).bfloat16())
+            st["v"].copy_(torch.randn(b, L, d, generator=gen).bfloat16())
+            st["lr1"].copy_(torch.nn.functional.softplus(torch.randn(b, L, 1, generator=gen) - 3.0))
+        graph.replay()
+        torch.cuda.synchronize()
+        out_r, grads_r = out_g.clone(), {n: g.clone() for n, g in grads_g.items()}
+        out_e, grads_e = run()
+        torch.cuda.synchronize()
+        assert torch.equal(out_r, out_e), rep
+        for n in grads_e:
+            assert torch.equal(grads_r[n], grads_e[n]), (rep, n)
+
+
 def test_calls_on_two_caller_streams():
     """Two independent problems enqueued on two caller streams at once (forward and backward each), as a caller with
     its own stream pool would: the library's side streams, the ordering of the fused Newton-Schulz kernels across
