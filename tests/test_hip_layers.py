@@ -268,3 +268,55 @@ def test_nvs_layer_against_oracle(steps):
     say("  ", errs)
     assert res["y1"].shape == (2, 100, 256) and res["y2"].shape == (2, 72, 256)
     assert max(errs.values()) < 1e-3
+
+
+def test_bidirectional_and_nvs_layers_bf16_autocast():
+    """The two other layers under bf16 autocast (projections and operation in bf16, rates in fp32), against the
+    oracle layers under the same policy on the CPU."""
+    say("bidirectional + nvs layers bf16 autocast")
+    torch.manual_seed(15)
+    kw = dict(dim=256, head_dim=128, inter_multi=1, use_muon=False)
+    ref_layer = LO.BidirectionalLaCTSwiGLU(num=AC, **kw)
+    layer = HL.BidirectionalLaCTSwiGLU(**kw).to(DEV)
+    layer.load_state_dict(ref_layer.state_dict(), strict=True)
+    x, go = torch.randn(2, 300, 256), torch.randn(2, 300, 256)
+    with torch.autocast("cpu", dtype=torch.bfloat16):
+        ref = grads_and_out(ref_layer, x, go)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        res = grads_and_out(layer, x.to(DEV), go.to(DEV))
+    errs = compare(res, ref)
+    say("  ", errs)
+    assert max(errs.values()) < 3e-2
+
+    kw = dict(dim=256, head_dim=128, inter_multi=2, bias=True, muon_update_steps=0)
+    ref_nvs = LO.FastWeightGluMLPMultihead(num=AC, **kw)
+    nvs_layer = HL.FastWeightGluMLPMultihead(**kw).to(DEV)
+    nvs_layer.load_state_dict(ref_nvs.state_dict(), strict=True)
+    order = [O.TTTOperator(0, 200, True, False), O.TTTOperator(200, 300, False, True)]
+    with torch.autocast("cpu", dtype=torch.bfloat16), torch.no_grad():
+        y_ref, st_ref = ref_nvs(x, {"ttt_op_order": order})
+    with torch.autocast("cuda", dtype=torch.bfloat16), torch.no_grad():
+        y, st = nvs_layer(x.to(DEV), {"ttt_op_order": order})
+    e = {"y": O.rel_l2(y.float().cpu(), y_ref.float()), **{n: O.rel_l2(st[n].float().cpu(), st_ref[n].float()) for n in st}}
+    say("  ", e)
+    assert y.shape == (2, 100, 256) and max(e.values()) < 3e-2
+
+
+def test_layer_under_activation_checkpointing():
+    """torch.utils.checkpoint runs the layer's forward a second time inside the backward (lact_nvs/train.py:106-123
+    wraps its blocks that way): same output and gradients as the plain call."""
+    say("layer under activation checkpointing")
+    from torch.utils.checkpoint import checkpoint
+    torch.manual_seed(16)
+    layer = HL.CausalLaCTSwiGLUWithSlidingWindowAttn(dim=256, head_dim=128, attn_head_dim=64, lact_chunk_size=128,
+                                                     window_size=64, use_muon=True).to(DEV)
+    x = torch.randn(2, 3 * 128 + 17, 256, device=DEV)
+    go = torch.randn_like(x)
+    plain = grads_and_out(layer, x, go)
+    xc = x.clone().requires_grad_(True)
+    y = checkpoint(layer, xc, use_reentrant=False)
+    y.backward(go)
+    assert torch.equal(y.detach().float().cpu(), plain["y"])
+    assert torch.equal(xc.grad.float().cpu(), plain["dx"])
+    for n, p in layer.named_parameters():
+        assert torch.equal(p.grad.detach().float().cpu(), plain["d." + n]), n
