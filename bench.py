@@ -48,6 +48,11 @@ MEASURED_TRAFFIC_MIB = {
 }
 
 
+# Whole step at config 1, same two counter runs (last line of that profile): read + written MiB
+MEASURED_STEP_TRAFFIC_MIB = 2930.0 + 1676.0
+PEAK_HBM_GBPS = 8000.0
+
+
 def algorithmic_flops(b, L, d, dh, C, ns_steps=5):
     """Counted FLOPs of fwd+bwd (multiply-add = 2; backward = 2x forward; recompute, momentum, renorm and
     pointwise work not counted): F_apply = 6 d dh T, F_update = 12 d dh T, F_ns = 3 steps (4 r^2 c + 2 r^3)."""
@@ -182,6 +187,11 @@ def main():
               "tflops": (r["flops"] / (r["ms"] * 1e-3) / 1e12) if r["ms"] > 0 and r["flops"] > 0 else None}
              for r in rows], key=lambda r: -r["ms_per_step"])
         res["kernel_ms_per_step"] = total_ms / args.steps
+    if args.config == "c1":
+        gbps = MEASURED_STEP_TRAFFIC_MIB * 2 ** 20 / (ms_per_step * 1e-3) / 1e9
+        res["step_hbm"] = {"bytes_per_step": MEASURED_STEP_TRAFFIC_MIB * 2 ** 20, "achieved": gbps, "peak": PEAK_HBM_GBPS,
+                           "unit": "GB/s", "frac": gbps / PEAK_HBM_GBPS,
+                           "source": "profiles/c1_fwd_bwd_hbm_traffic_pmc.txt (FETCH_SIZE + WRITE_SIZE of every kernel of a step)"}
 
     # ---- CPU baseline: the oracle (a restatement of the reference's non-fused PyTorch op) on the host cores
     if not args.no_cpu_baseline:
