@@ -20,10 +20,9 @@ import numpy as np
 import pytest
 import torch
 
-import lact_amd
 from lact_amd import ar_video, minimal, nvs, ops
 from lact_amd import ttt_operation as T
-from lact_amd._lib import LACT_APPLY, LACT_UPDATE
+from lact_amd._lib import LACT_APPLY
 from oracle import lact_oracle as O
 
 pytestmark = pytest.mark.gpu

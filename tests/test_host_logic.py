@@ -3,7 +3,6 @@
 import os
 import subprocess
 
-import pytest
 
 from lact_amd import _lib
 

@@ -1,7 +1,6 @@
 """Pins the CPU restatement of the layer classes (oracle/lact_layers_oracle.py): golden vectors written from the
 reference's own BidirectionalLaCTSwiGLU on the CPU (tests/golden/bidirectional_layer_cpu_fp32.npz), and
 closed-form checks for what the causal layer adds (attention window, per-head gate, momentum head, q/k rescale)."""
-import math
 import os
 
 import numpy as np
