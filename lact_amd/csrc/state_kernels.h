@@ -329,9 +329,21 @@ __global__ void k_renorm_bwd(const RenormParams p) {
   float c0 = 1.f, c1 = 0.f;
   float* gn0 = p.gn0 + (size_t)z * p.g.maxrows() + row;
   if (!p.weight_norm && p.gn0_init && lane == 0) *gn0 = 0.f;
+  // the first 1024 columns of a row stay in registers between the two passes (as in k_update_renorm)
+  float4 wv[ROW_VEC_MAX], gk[ROW_VEC_MAX];
   if (p.weight_norm) {
     float ss = 0.f, dot = 0.f;
-    for (int c = lane * 4; c < cols; c += 256) {
+#pragma unroll
+    for (int i = 0; i < ROW_VEC_MAX; ++i) {
+      const int c = lane * 4 + i * 256;
+      if (c < cols) {
+        wv[i] = renorm_w_hat4(p, o + c, uo + c);
+        gk[i] = renorm_gy4(p, o + c);
+        ss += dot4(wv[i], wv[i]);
+        if (p.gy || p.gy2) dot += dot4(wv[i], gk[i]);
+      }
+    }
+    for (int c = lane * 4 + ROW_VEC_MAX * 256; c < cols; c += 256) {
       const float4 v = renorm_w_hat4(p, o + c, uo + c);
       ss += dot4(v, v);
       if (p.gy || p.gy2) dot += dot4(v, renorm_gy4(p, o + c));
@@ -351,11 +363,9 @@ __global__ void k_renorm_bwd(const RenormParams p) {
       if (lane == 0) *gn0 = (p.gn0_init ? 0.f : *gn0) + dot / (r + 1e-5f);
     }
   }
-  for (int c = lane * 4; c < cols; c += 256) {
-    float4 gv = renorm_gy4(p, o + c);
+  auto emit = [&](int c, float4 gv, const float4& w) {
     gv = f4(gv.x * c0, gv.y * c0, gv.z * c0, gv.w * c0);
     if (p.weight_norm) {
-      const float4 w = renorm_w_hat4(p, o + c, uo + c);
       gv.x -= w.x * c1; gv.y -= w.y * c1; gv.z -= w.z * c1; gv.w -= w.w * c1;
     }
     if (p.carry_in) {
@@ -379,7 +389,18 @@ __global__ void k_renorm_bwd(const RenormParams p) {
         }
       }
     }
+  };
+  const float4 zero4 = f4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+  for (int i = 0; i < ROW_VEC_MAX; ++i) {
+    const int c = lane * 4 + i * 256;
+    if (c < cols) {
+      if (p.weight_norm) emit(c, gk[i], wv[i]);
+      else emit(c, renorm_gy4(p, o + c), zero4);
+    }
   }
+  for (int c = lane * 4 + ROW_VEC_MAX * 256; c < cols; c += 256)
+    emit(c, renorm_gy4(p, o + c), p.weight_norm ? renorm_w_hat4(p, o + c, uo + c) : zero4);
 }
 
 // ---- backward of the Frobenius normalisation, the momentum recurrence and the raw-gradient add --
