@@ -151,8 +151,8 @@ int lact_layer_post_backward(int32_t act_dtype, int32_t B, int32_t L, int32_t H,
  *     use) that are forked from and joined back into the caller's stream with events, so the call as a whole
  *     stays asynchronous and ordered on the caller's stream.
  *   LACT_OPT_FUSED_NEWTON_SCHULZ: all Newton-Schulz iterations of an update (and of its backward) run as one
- *     kernel whose blocks meet at per-matrix barriers (bf16, rows and columns multiples of 192 or of 128, at most 8
- *     iterations); otherwise three GEMM launches per iteration.
+ *     kernel whose blocks meet at per-matrix barriers (bf16; rows and columns multiples of 192, of 128, or rows of
+ *     128 and columns of 64; at most 8 iterations); otherwise three GEMM launches per iteration.
  * Returns the previous value (0 / 1), or -1 for an unknown option. */
 enum { LACT_OPT_STREAM_OVERLAP = 0, LACT_OPT_FUSED_NEWTON_SCHULZ = 1 };
 int lact_set_option(int32_t option, int32_t value);

@@ -447,16 +447,27 @@ struct Runner {
     if (side && g_overlap) { s_side = side->stream; s_tail = side->tail; }
   }
   // ---- fused Newton-Schulz: launches of at most 256 resident blocks
-  static bool tiles_fit(int r, int c, int edge) { return r % edge == 0 && c % edge == 0 && (r / edge) * (c / edge) <= 32; }
-  // 192 x 192 tiles when the matrices fill at least half the chip with them, else 128 x 128 (more, smaller blocks)
-  static bool ns_fused_small_tiles(const NsBatch& B) {
-    if (!tiles_fit(B.r, B.c, 128)) return false;
-    if (!tiles_fit(B.r, B.c, 192)) return true;
-    return B.n * (B.r / 192) * (B.c / 192) < 128;
+  static bool tiles_fit(int r, int c, int bm, int bn) {
+    return r % bm == 0 && r % bn == 0 && c % bn == 0 && (r / bm) * (c / bn) <= 32;
+  }
+  // Tile of the fused kernel for a batch: 0 = 192 x 192, 1 = 128 x 128, 2 = 128 x 64, -1 = none fits.
+  // 192 x 192 when the matrices fill at least half the chip with it, else 128 x 128 (more, smaller blocks), and
+  // 128 x 64 when even those leave most of the chip idle -- as long as the groups dealt to one XCD (a matrix's
+  // blocks share an XCD) still find a compute unit each there.
+  static int ns_fused_tile(const NsBatch& B) {
+    const bool f192 = tiles_fit(B.r, B.c, 192, 192), f128 = tiles_fit(B.r, B.c, 128, 128), f64 = tiles_fit(B.r, B.c, 128, 64);
+    if (f192 && (!f128 || B.n * (B.r / 192) * (B.c / 192) >= 128)) return 0;
+    const int per_xcd = (B.n + 7) / 8;
+    if (f64) {
+      const int nbm64 = (B.r / 128) * (B.c / 64);
+      if (per_xcd * nbm64 <= 32 && (!f128 || B.n * (B.r / 128) * (B.c / 128) < 128)) return 2;
+    }
+    if (f128) return 1;
+    return f192 ? 0 : -1;
   }
   bool ns_fused_ok(const NsBatch& B) const {
     if (!g_fused_ns || !side || !kNsBf16 || P.S < 1 || P.S > NS_FUSED_MAX_STEPS) return false;
-    return tiles_fit(B.r, B.c, 192) || tiles_fit(B.r, B.c, 128);
+    return ns_fused_tile(B) >= 0;
   }
   bool ns_fused_any() const {
     for (auto& B : P.nsb)
@@ -497,8 +508,12 @@ struct Runner {
   }
   template <bool BWD>
   void launch_ns_fused(const NsFusedParams& p, const NsBatch& B) {
-    if (ns_fused_small_tiles(B)) launch_ns_fused_ts<TS_SQ, BWD>(p, B);
-    else launch_ns_fused_ts<TS_NS, BWD>(p, B);
+    switch (ns_fused_tile(B)) {
+      case 0: launch_ns_fused_ts<TS_NS, BWD>(p, B); break;
+      case 1: launch_ns_fused_ts<TS_SQ, BWD>(p, B); break;
+      case 2: launch_ns_fused_ts<TS_BWD, BWD>(p, B); break;
+      default: break;
+    }
   }
   // `waiter` waits for everything enqueued so far on `on`
   void wait_for(hipStream_t waiter, hipStream_t on) {

@@ -102,20 +102,20 @@ __device__ __forceinline__ void ns_term(RowGemmTerm& t, const void* A, int lda, 
 
 // BWD = false: S iterations  A = X X^T;  B = b A + c A A;  X' = a X + B X
 // BWD = true:  the same iterations backwards:  Sg = G X^T + X G^T;  H = b Sg + c (Sg A + A Sg);  G' = a G + B G + H X
-// TS: 192 x 192 tiles, or 128 x 128 when there are too few matrices to fill the chip with the large tile.
+// TS: 192 x 192 tiles, or 128 x 128 / 128 x 64 when there are too few matrices to fill the chip with the large tile.
 template <class TS, bool BWD>
 __global__ __launch_bounds__(DMA_THREADS) void k_ns_fused(const NsFusedParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  const int tr = p.r / TS::BM, tc = p.c / TS::BN;
-  const int nbm = tr * tc;                           // blocks per matrix
+  const int tr = p.r / TS::BM, tc = p.c / TS::BN, ts = p.r / TS::BN;   // tile rows; tile columns of [r, c] and of [r, r]
+  const int nbm = tr * tc;                           // blocks per matrix (c >= r: the r x c stages have the most tiles)
   const int L = blockIdx.x, j = L >> 3;
   const int group = (L & 7) + 8 * (j / nbm), member = j % nbm;
   if (group >= p.n) return;
   const int z = p.z0 + group;
   GroupBarrier bar;
   bar.init(p.sync + (size_t)group * 32, nbm, p.error);
-  const bool sq_tile = member < tr * tr;             // this block owns a tile of the r x r stages
-  const int sx = member / tr, sy = member % tr;      // its tile there
+  const bool sq_tile = member < tr * ts;             // this block owns a tile of the r x r stages
+  const int sx = member / ts, sy = member % ts;      // its tile there
   const int rx = member / tc, ry = member % tc;      // its tile of the r x c stages
 
   LACT_NS_TS(0);
