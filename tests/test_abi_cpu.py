@@ -76,6 +76,14 @@ def test_query_sizes_and_validation_messages():
     assert "ns_coeffs" in err(make_desc(ops.block_causal_steps(256, 64), ns_steps=5))
     assert "alignment" in err(make_desc(ops.block_causal_steps(256, 64), q_ld=68))
     assert "act_dtype" in err(make_desc(ops.block_causal_steps(256, 64), act_dtype=3))
+    # a forward-only descriptor keeps less for the backward, and the backward entry point refuses it (before it
+    # looks at any pointer: no GPU is needed for this check)
+    rc, saved_fo, _ = sizes(make_desc(ops.block_causal_steps(256, 64), forward_only=1))
+    assert rc == 0 and saved_fo < saved
+    null = ctypes.c_void_p(0)
+    fo = make_desc(ops.block_causal_steps(256, 64), forward_only=1)
+    assert L.lact_backward(ctypes.byref(fo), *([null] * 22)) != 0
+    assert "forward_only" in L.lact_last_error().decode()
     assert L.lact_query_sizes(None, None, None) != 0 and "null" in L.lact_last_error().decode()
     assert L.lact_newton_schulz_workspace_bytes(4, 64, 128, 5) > 0
     assert L.lact_newton_schulz_workspace_bytes(0, 64, 128, 5) == 0

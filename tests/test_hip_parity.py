@@ -470,6 +470,31 @@ def test_config4_full_size_properties():
     full_size_properties(12, 32760, 128, 256, 4680, 1004, False)
 
 
+def test_forward_only_and_output_only_calls():
+    """Under torch.no_grad the descriptor is forward-only (nothing kept for a backward) and the output has the same
+    bits as in a training call; a program with return_state=False returns None for the final weights and momentum
+    states, with the same output."""
+    say("forward-only / output-only")
+    b, L, d, dh, C = 2, 3 * 128 + 9, 128, 128, 128
+    inp = problem(b, L, d, dh, seed=31, act=torch.bfloat16)
+    t = clone_to(inp, DEV)
+    out_train = T.block_causal_lact_swiglu(*args9(t), C, True, t["momentum"])
+    with torch.no_grad():
+        out_infer = T.block_causal_lact_swiglu(*args9(t), C, True, t["momentum"])
+    assert torch.equal(out_train, out_infer) and not out_infer.requires_grad
+    steps = ops.block_causal_steps(L, C)
+    full = ops.Program(steps=steps, out_len=L, ns_coeffs=ops.NS5_COEFFS)
+    lean = ops.Program(steps=steps, out_len=L, ns_coeffs=ops.NS5_COEFFS, return_state=False)
+    o1, w1, m1 = ops.run_program(full, *args9(t), t["momentum"])
+    o2, w2, m2 = ops.run_program(lean, *args9(t), t["momentum"])
+    assert torch.equal(o1, o2) and torch.equal(o1, out_train)
+    assert all(w is not None for w in w1) and all(m is not None for m in m1)
+    assert all(w is None for w in w2) and all(m is None for m in m2)
+    g1 = grads_of(o1, t, torch.ones_like(o1))
+    g2 = grads_of(o2, t, torch.ones_like(o2))
+    assert all(torch.equal(g1[n], g2[n]) for n in g1)
+
+
 def test_graph_capture_replays_match_eager():
     """Forward + backward captured into a HIP graph (the library forks and joins its side streams with events
     only, and clears memory with kernels): three replays on fresh inputs, with eager work and synchronisations in
