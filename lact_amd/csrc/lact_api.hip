@@ -469,6 +469,13 @@ struct Runner {
     if (!g_fused_ns || !side || !kNsBf16 || P.S < 1 || P.S > NS_FUSED_MAX_STEPS) return false;
     return ns_fused_tile(B) >= 0;
   }
+  // every batch runs fused (and at least one iteration): the Frobenius normalisation is the fused kernel's first stage
+  bool ns_all_fused() const {
+    if (!P.muon || P.nsb.empty()) return false;
+    for (auto& B : P.nsb)
+      if (!ns_fused_ok(B)) return false;
+    return true;
+  }
   bool ns_fused_any() const {
     for (auto& B : P.nsb)
       if (ns_fused_ok(B)) return true;
@@ -777,18 +784,22 @@ struct Runner {
         p.round_partial_bf16 = P.bf16;
         if (u + 1 == P.nupd && P.momentum && m_out)
           for (int j = 0; j < 3; ++j) p.m_ext[j] = m_out[j];
+        if (ns_all_fused()) p.clear = ns_clear();
         LACT_LAUNCH("k_momentum_prep", "k_momentum_prep", 0.0, (k_momentum_prep<TN>), dim3(P.nblk, 3 * d.b), dim3(256), s, p);
       }
       flush_applies(true);
       if (P.muon) {
-        NsScaleParams p;
-        memset(&p, 0, sizeof(p));
-        p.g = P.g; p.g16 = g16(u); p.ss_part = scr<float>(P.t_ss); p.nparts = P.nblk; p.norms = norms(u);
-        p.xf = scr<float>(P.t_xf[0]); p.xb = xb(u, 0);
-        p.u = P.S == 0 ? usave(u) : nullptr;
-        p.plain_bf16 = d.ns_mode == LACT_NS_PLAIN_BF16;
-        p.clear = ns_clear();
-        LACT_LAUNCH("k_ns_scale", "k_ns_scale", 0.0, (k_ns_scale<TN>), dim3(P.nblk, P.g.ns_count()), dim3(256), s, p);
+        const bool scale_in_kernel = ns_all_fused();
+        if (!scale_in_kernel) {
+          NsScaleParams p;
+          memset(&p, 0, sizeof(p));
+          p.g = P.g; p.g16 = g16(u); p.ss_part = scr<float>(P.t_ss); p.nparts = P.nblk; p.norms = norms(u);
+          p.xf = scr<float>(P.t_xf[0]); p.xb = xb(u, 0);
+          p.u = P.S == 0 ? usave(u) : nullptr;
+          p.plain_bf16 = d.ns_mode == LACT_NS_PLAIN_BF16;
+          p.clear = ns_clear();
+          LACT_LAUNCH("k_ns_scale", "k_ns_scale", 0.0, (k_ns_scale<TN>), dim3(P.nblk, P.g.ns_count()), dim3(256), s, p);
+        }
         for (const NsBatch& B : P.nsb) {
           if (ns_fused_ok(B)) {
             if constexpr (kNsBf16) {
@@ -799,6 +810,12 @@ struct Runner {
               f.xb = xb(u, 0) + B.xoff; f.xb_it_stride = (long long)P.mat3;
               f.ab = ab(u, 0) + B.sqoff; f.bb = bb(u, 0) + B.sqoff; f.sq_it_stride = (long long)sq3();
               f.xb_last = scr<uint16_t>(P.t_xbtmp) + B.xoff; f.u_out = usave(u) + B.xoff;
+              if (scale_in_kernel) {
+                f.g16 = reinterpret_cast<const uint16_t*>(g16(u)) + B.xoff;
+                f.ss_part = scr<float>(P.t_ss); f.nparts = P.nblk;
+                f.part0 = B.first; f.part1 = (P.g.stacked && B.first == 0) ? 2 * d.b : -1;
+                f.norms = norms(u) + B.first;
+              }
               launch_ns_fused<false>(f, B);
             }
             continue;

@@ -47,6 +47,10 @@ struct NsFusedParams {
   float* u_out;                                    // X_S, fp32, original orientation
   // backward: incoming gradient in gxf[0] / gxb[0]; the result ends in gxf[S & 1]
   float* gxf[2]; uint16_t* gxb[2]; uint16_t* sg; uint16_t* gas;
+  // forward, optional first stage: X_0 = G / (|G|_F + 1e-7) from the bf16 gradient g16 (laid out like xb) and the
+  // partial sums of its squares; writes xf[0], xb (iteration 0) and the norms.  Null g16: X_0 is there already.
+  const uint16_t* g16; const float* ss_part; int nparts, part0, part1;   // partial rows part0 + z and (if >= 0) part1 + z
+  float* norms;              // [n] of this batch
   unsigned* sync;            // [n][32] words, zeroed before the launch: word 0 = arrivals, word 1 = XCC id mask
   unsigned* error;           // set to 1 by a block whose barrier timed out
 };
@@ -118,6 +122,42 @@ __global__ __launch_bounds__(DMA_THREADS) void k_ns_fused(const NsFusedParams p)
   const int sx = member / ts, sy = member % ts;      // its tile there
   const int rx = member / tc, ry = member % tc;      // its tile of the r x c stages
 
+  if (!BWD && p.g16) {
+    // Frobenius normalisation in front of the first iteration: every block of the group sums the same partials
+    // in the same order, then scales its own tile of [r, c]
+    float ss = 0.f;
+    for (int i = 0; i < p.nparts; ++i) ss += p.ss_part[(size_t)(p.part0 + z) * p.nparts + i];
+    if (p.part1 >= 0)
+      for (int i = 0; i < p.nparts; ++i) ss += p.ss_part[(size_t)(p.part1 + z) * p.nparts + i];
+    float n = sqrtf(ss);
+    if (p.plain) n = round_bf16(n);
+    if (member == 0 && threadIdx.x == 0) p.norms[z] = n;
+    float den = n + 1e-7f;
+    if (p.plain) den = round_bf16(den);
+    const float inv = 1.f / den;
+    const size_t zo = (size_t)z * p.r * p.c + (size_t)rx * TS::BM * p.c + ry * TS::BN;
+    constexpr int GR = TS::BN / 8;   // 16-byte granules per tile row
+    for (int id = threadIdx.x; id < TS::BM * GR; id += DMA_THREADS) {
+      const size_t o = zo + (size_t)(id / GR) * p.c + (id % GR) * 8;
+      const uint4 u = *reinterpret_cast<const uint4*>(p.g16 + o);
+      const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+      float v[8];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __uint_as_float(w[i] << 16) * inv;
+        v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u) * inv;
+      }
+      if (p.plain) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = round_bf16(v[i]);
+      }
+      *reinterpret_cast<float4*>(p.xf[0] + o) = make_float4(v[0], v[1], v[2], v[3]);
+      *reinterpret_cast<float4*>(p.xf[0] + o + 4) = make_float4(v[4], v[5], v[6], v[7]);
+      Elem<uint16_t>::store4(p.xb + o, v[0], v[1], v[2], v[3]);
+      Elem<uint16_t>::store4(p.xb + o + 4, v[4], v[5], v[6], v[7]);
+    }
+    bar.sync(p.error);
+  }
   LACT_NS_TS(0);
   for (int step = 0; step < p.S; ++step) {
     const int it = BWD ? p.S - 1 - step : step;

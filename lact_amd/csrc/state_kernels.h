@@ -126,11 +126,13 @@ struct MomentumPrepParams {
   void* g16;                          // [3b][elems]  d_out cast to the Newton-Schulz type, in its orientation, or null
   float* ss_part;                     // [3b][gridDim.x]
   int round_partial_bf16;             // the reduction GEMM's result is a bf16 tensor in the reference
+  ClearWords clear;
 };
 template <typename TN>
 __global__ void k_momentum_prep(const MomentumPrepParams p) {
   __shared__ float red[16];
   const int z = blockIdx.y, j = z / p.g.nb, ib = z % p.g.nb;
+  clear_words(p.clear, blockIdx.x == 0 && blockIdx.y == 0);
   const FlatRange R(p.g.elems);
   const float mb = (p.m_prev && p.mbar) ? p.mbar[ib] : 0.f;
   const size_t zo = (size_t)z * p.g.elems, stride = (size_t)3 * p.g.nb * p.g.elems;
