@@ -306,7 +306,7 @@ struct Plan {
     for (int i = 0; i < 2; ++i) t_xf[i] = sc.take(mat3 * 4);
     t_xbtmp = sc.take(mat3 * nsz);
     t_ss = sc.take((size_t)3 * d.b * nblk * 4);
-    t_dot = sc.take((size_t)3 * d.b * nblk * 4);
+    t_dot = sc.take((size_t)3 * d.b * std::max(nblk, 32) * 4);   // partial dots: per chunk of a matrix, or per block of the fused kernel
     t_mdot = sc.take((size_t)3 * d.b * nblk * 4);
     for (int i = 0; i < 2; ++i) t_gwhat[i] = sc.take(mat3 * 4);
     t_gwcur = sc.take(mat3 * 4);
@@ -464,6 +464,14 @@ struct Runner {
     }
     if (f128) return 1;
     return f192 ? 0 : -1;
+  }
+  static int ns_fused_nbm(const NsBatch& B) {   // blocks per matrix of the fused kernel
+    switch (ns_fused_tile(B)) {
+      case 0: return (B.r / 192) * (B.c / 192);
+      case 1: return (B.r / 128) * (B.c / 128);
+      case 2: return (B.r / 128) * (B.c / 64);
+      default: return 0;
+    }
   }
   bool ns_fused_ok(const NsBatch& B) const {
     if (!g_fused_ns || !side || !kNsBf16 || P.S < 1 || P.S > NS_FUSED_MAX_STEPS) return false;
@@ -1092,7 +1100,15 @@ struct Runner {
         }
       }
       if (d.prenorm) carry_main = gw_idx;
+      // The backward of the Frobenius normalisation as the fused kernel's last stages: the partial dots always
+      // (one batch, every matrix fused); the gradient in the compute type too when nothing else enters it (no
+      // momentum state to carry, no raw-gradient term) and every matrix is held as it lies (square shapes).
+      const bool dot_in_kernel = ns_all_fused() && P.nsb.size() == 1;
+      const bool carry_here = P.momentum && (u > 0 || gm_valid);
+      const bool prep_in_kernel = dot_in_kernel && kBf16 && !carry_here && !(P.muon && d.muon_replaces_weight) &&
+                                  P.g.x_contiguous(0) && P.g.x_contiguous(1) && P.g.x_contiguous(2);
       if (P.muon) {
+        if (prep_in_kernel) wait_tail();   // the previous update's dk GEMM reads the gradient copy the fused kernel writes
         for (const NsBatch& B : P.nsb) {
           const int n = B.n, r = B.r, c = B.c;
           const long long xe = (long long)r * c, se = (long long)r * r;
@@ -1107,6 +1123,12 @@ struct Runner {
               f.gxf[0] = scr<float>(P.t_gxf[0]) + B.xoff; f.gxf[1] = scr<float>(P.t_gxf[1]) + B.xoff;
               f.gxb[0] = scr<uint16_t>(P.t_gxb[0]) + B.xoff; f.gxb[1] = scr<uint16_t>(P.t_gxb[1]) + B.xoff;
               f.sg = reinterpret_cast<uint16_t*>(sg); f.gas = reinterpret_cast<uint16_t*>(gas);
+              if (dot_in_kernel) {
+                f.g16 = reinterpret_cast<const uint16_t*>(g16(u)) + B.xoff;
+                f.dot_part = scr<float>(P.t_dot);
+                f.norms = norms(u) + B.first;
+                if (prep_in_kernel) f.gc = scr<uint16_t>(P.t_gc) + B.xoff;
+              }
               launch_ns_fused<true>(f, B);
             }
             continue;
@@ -1148,17 +1170,19 @@ struct Runner {
           }
         }
         cur = P.S & 1;
-        NsDotParams dp;
-        dp.g = P.g; dp.gx0 = scr<float>(P.t_gxf[cur]); dp.g16 = g16(u); dp.dot_part = scr<float>(P.t_dot);
-        LACT_LAUNCH("k_ns_bwd_dot", "k_ns_bwd_dot", 0.0, (k_ns_bwd_dot<TN>), dim3(P.nblk, P.g.ns_count()), dim3(256), s, dp);
+        if (!dot_in_kernel) {
+          NsDotParams dp;
+          dp.g = P.g; dp.gx0 = scr<float>(P.t_gxf[cur]); dp.g16 = g16(u); dp.dot_part = scr<float>(P.t_dot);
+          LACT_LAUNCH("k_ns_bwd_dot", "k_ns_bwd_dot", 0.0, (k_ns_bwd_dot<TN>), dim3(P.nblk, P.g.ns_count()), dim3(256), s, dp);
+        }
       }
-      {
+      if (!(P.muon && prep_in_kernel)) {
         wait_tail();   // the previous update's dk GEMM reads the gradient copy written here
         GradPrepParams p;
         memset(&p, 0, sizeof(p));
         p.g = P.g; p.muon = P.muon;
         p.gx0 = scr<float>(P.t_gxf[cur]); p.g16 = P.muon ? (const void*)g16(u) : nullptr; p.norms = norms(u);
-        p.dot_part = scr<float>(P.t_dot); p.nparts = P.nblk;
+        p.dot_part = scr<float>(P.t_dot); p.nparts = (P.muon && dot_in_kernel) ? ns_fused_nbm(P.nsb[0]) : P.nblk;
         p.gw_hat = gwhat; p.cr = (P.muon && d.muon_replaces_weight) ? 1.f : 0.f;
         p.gm_carry = (P.momentum && (u > 0 || gm_valid)) ? gmcarry : nullptr; p.carry_valid = gm_valid;
         p.carry_write = u > 0;
@@ -1174,6 +1198,8 @@ struct Runner {
             LACT_LAUNCH("k_momentum_grad", "k_momentum_grad", 0.0, k_momentum_grad, dim3(d.b), dim3(256), s, scr<float>(P.t_mdot), P.nblk, d.b, dmom,
                                (long long)d.kv_len, st.start, T_);
         }
+      } else if (P.momentum) {
+        gm_valid = true;   // nothing was carried (first update of the program): as after the kernel above
       }
       const T* kc = k + (size_t)st.start * d.k_ld;
       const T* vc = v + (size_t)st.start * d.v_ld;

@@ -51,6 +51,11 @@ struct NsFusedParams {
   // partial sums of its squares; writes xf[0], xb (iteration 0) and the norms.  Null g16: X_0 is there already.
   const uint16_t* g16; const float* ss_part; int nparts, part0, part1;   // partial rows part0 + z and (if >= 0) part1 + z
   float* norms;              // [n] of this batch
+  // backward, optional last stages (the backward of that normalisation): every block writes <G_final, g16> over
+  // its tile to dot_part[z][member]; with gc set, the blocks then meet once more and each writes its tile of
+  //   gc = G_final / (n + 1e-7) - g16 * <G_final, g16> / (n (n + 1e-7)^2)
+  // (the gradient w.r.t. the Newton-Schulz input in the compute type; norms as written by the forward)
+  float* dot_part; uint16_t* gc;
   unsigned* sync;            // [n][32] words, zeroed before the launch: word 0 = arrivals, word 1 = XCC id mask
   unsigned* error;           // set to 1 by a block whose barrier timed out
 };
@@ -243,6 +248,55 @@ __global__ __launch_bounds__(DMA_THREADS) void k_ns_fused(const NsFusedParams p)
       LACT_NS_TS(1 + step * 6 + 4);
       bar.sync(p.error);
       LACT_NS_TS(1 + step * 6 + 5);
+    }
+  }
+  if (BWD && p.dot_part) {
+    // the tile this block wrote in the last stage, and the same tile of the bf16 input: 12 granules of 8 elements
+    // per thread at 192 x 192, kept in registers for the second pass
+    constexpr int GR = TS::BN / 8, NG = (TS::BM * GR + DMA_THREADS - 1) / DMA_THREADS;
+    const float* gx = p.gxf[p.S & 1];
+    const size_t zo = (size_t)z * p.r * p.c + (size_t)rx * TS::BM * p.c + ry * TS::BN;
+    float4 ga[NG], gb[NG];
+    uint4 gi[NG];
+    float dot = 0.f;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");   // the vector L1 may hold this buffer's lines from two iterations ago
+#pragma unroll
+    for (int t = 0; t < NG; ++t) {
+      const int id = threadIdx.x + t * DMA_THREADS;
+      if (id < TS::BM * GR) {
+        const size_t o = zo + (size_t)(id / GR) * p.c + (id % GR) * 8;
+        ga[t] = *reinterpret_cast<const float4*>(gx + o);
+        gb[t] = *reinterpret_cast<const float4*>(gx + o + 4);
+        gi[t] = *reinterpret_cast<const uint4*>(p.g16 + o);
+        const uint32_t w[4] = {gi[t].x, gi[t].y, gi[t].z, gi[t].w};
+        dot += ga[t].x * __uint_as_float(w[0] << 16) + ga[t].y * __uint_as_float(w[0] & 0xffff0000u) +
+               ga[t].z * __uint_as_float(w[1] << 16) + ga[t].w * __uint_as_float(w[1] & 0xffff0000u) +
+               gb[t].x * __uint_as_float(w[2] << 16) + gb[t].y * __uint_as_float(w[2] & 0xffff0000u) +
+               gb[t].z * __uint_as_float(w[3] << 16) + gb[t].w * __uint_as_float(w[3] & 0xffff0000u);
+      }
+    }
+    dot = block_sum(dot, reinterpret_cast<float*>(smem));
+    if (threadIdx.x == 0) p.dot_part[(size_t)z * nbm + member] = dot;
+    if (p.gc) {
+      bar.sync(p.error);
+      float total = 0.f;
+      for (int i = 0; i < nbm; ++i) total += __hip_atomic_load(p.dot_part + (size_t)z * nbm + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const float n = p.norms[z];
+      float c0 = 1.f / (n + 1e-7f);
+      const float c1 = n > 0.f ? total / (n * (n + 1e-7f) * (n + 1e-7f)) : 0.f;
+      if (__hip_atomic_load(p.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) c0 = __uint_as_float(0x7fc00000u);
+#pragma unroll
+      for (int t = 0; t < NG; ++t) {
+        const int id = threadIdx.x + t * DMA_THREADS;
+        if (id < TS::BM * GR) {
+          const size_t o = zo + (size_t)(id / GR) * p.c + (id % GR) * 8;
+          const uint32_t w[4] = {gi[t].x, gi[t].y, gi[t].z, gi[t].w};
+          Elem<uint16_t>::store4(p.gc + o, ga[t].x * c0 - __uint_as_float(w[0] << 16) * c1, ga[t].y * c0 - __uint_as_float(w[0] & 0xffff0000u) * c1,
+                                 ga[t].z * c0 - __uint_as_float(w[1] << 16) * c1, ga[t].w * c0 - __uint_as_float(w[1] & 0xffff0000u) * c1);
+          Elem<uint16_t>::store4(p.gc + o + 4, gb[t].x * c0 - __uint_as_float(w[2] << 16) * c1, gb[t].y * c0 - __uint_as_float(w[2] & 0xffff0000u) * c1,
+                                 gb[t].z * c0 - __uint_as_float(w[3] << 16) * c1, gb[t].w * c0 - __uint_as_float(w[3] & 0xffff0000u) * c1);
+        }
+      }
     }
   }
 }

@@ -643,8 +643,9 @@ def test_stream_overlap_is_bit_identical(prenorm):
 @pytest.mark.parametrize("b,d,dh", [(5, 384, 192), (2, 384, 384), (3, 256, 128)])
 def test_fused_newton_schulz_is_bit_identical(b, d, dh):
     """All Newton-Schulz iterations of an update as one kernel with per-matrix barriers (rows, columns multiples
-    of 192) against three GEMM launches per iteration: same tile code, same order, so the same bits -- forward
-    and backward, with the apply steps running beside them on the second stream."""
+    of 192) against three GEMM launches per iteration: same tile code, same order, so the same bits in the forward
+    (and in every Newton-Schulz iterate of the backward), with the apply steps running beside them on the second
+    stream."""
     say("fused Newton-Schulz on/off", b, d, dh)
     from lact_amd import _lib
     # (5, 384, 192): w1 is held transposed ([192, 384]), 15 matrices = a partial group of 8, 192-tiles;
@@ -672,8 +673,11 @@ def test_fused_newton_schulz_is_bit_identical(b, d, dh):
     for (o1, g1), (o0, g0) in zip(on, off):
         assert torch.isfinite(o1.float()).all()
         assert torch.equal(o1, o0)
+        # backward: the fused kernel also sums the dot product of the normalisation's backward over its own tiles
+        # (the separate kernel sums it over flat chunks): fp32 sums in another order, nothing else differs
         for n in g0:
-            assert torch.equal(g1[n], g0[n]), n
+            assert O.rel_l2(g1[n], g0[n]) < 2e-3 and torch.isfinite(g1[n].float()).all(), n
+    assert all(torch.equal(on[0][1][n], on[1][1][n]) for n in on[0][1])     # and each path repeats its own bits
 
 
 # ---- fused-kernel variant (ttt_operation_fused_kernel.py): stacked Muon, eps inside the sqrt -------------
