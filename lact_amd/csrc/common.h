@@ -81,4 +81,14 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
   return t;
 }
 
+// Side job of a kernel that runs right before a fused Newton-Schulz launch: its first block clears the barrier
+// lines and the error word (a few KiB), which saves a launch of its own in the dependent chain.
+struct ClearWords {
+  unsigned* ptr; int n;
+};
+__device__ __forceinline__ void clear_words(const ClearWords& c, bool first_block) {
+  if (c.n > 0 && first_block)
+    for (int i = threadIdx.x; i < c.n; i += blockDim.x) c.ptr[i] = 0u;
+}
+
 }  // namespace lact

@@ -656,6 +656,7 @@ __global__ __launch_bounds__(DMA_THREADS) void k_token_reduce_dma(const TokenRed
   constexpr int STAGES = row_stages<TS>();
   using Pipe = DmaPipe<TS, 1, 2, STAGES>;
   int split, tile, bz;   // map: (splits, tiles, 3*nb)
+  clear_words(p.prep_clear, blockIdx.x == 0);
   if (!p.map.locate(blockIdx.x, split, tile, bz)) return;
   const int j = bz / p.nb, ib = bz % p.nb;
   const TokenReduceJob& job = p.job[j];
@@ -694,6 +695,47 @@ __global__ __launch_bounds__(DMA_THREADS) void k_token_reduce_dma(const TokenRed
   }
   __syncthreads();
   const size_t slot = (size_t)bz * p.mat_elems;
+  if (p.prep_d_out) {   // forward update, one split: momentum, bf16 copy and its sum of squares right here
+    const int r0 = ST::row0(), c0 = ST::col0();
+    float ss = 0.f;
+    if (ST::active() && n0 + c0 < job.N) {
+      const char* src = smem + (r0 * ST::LD + c0) * 4;
+      const size_t e0 = slot + (size_t)(m0 + r0) * job.N + n0 + c0, rstep = (size_t)ST::RPP * job.N;
+      const float mb = (p.prep_m_prev && p.prep_mbar) ? p.prep_mbar[ib] : 0.f;
+      float* ext = p.prep_m_ext[j] ? p.prep_m_ext[j] + (size_t)ib * p.mat_elems + (e0 - slot) : nullptr;
+      float4 x4[ST::PASSES];
+      if (p.prep_m_prev) {
+#pragma unroll
+        for (int ps = 0; ps < ST::PASSES; ++ps) {
+          const int r = r0 + ps * ST::RPP;
+          x4[ps] = (r < TS::BM && m0 + r < job.M) ? *reinterpret_cast<const float4*>(p.prep_m_prev + e0 + ps * rstep) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+      }
+      uint4 vg[8];
+#pragma unroll
+      for (int ps = 0; ps < ST::PASSES; ++ps) {
+        if (ps % 8 == 0) {
+#pragma unroll
+          for (int g = 0; g < 8; ++g)
+            if (ps + g < ST::PASSES) vg[g] = ST::read16(src, r0, ps + g);
+        }
+        const int r = r0 + ps * ST::RPP;
+        if (r < TS::BM && m0 + r < job.M) {
+          float4 v = __builtin_bit_cast(float4, vg[ps % 8]);
+          v = make_float4(round_bf16(v.x), round_bf16(v.y), round_bf16(v.z), round_bf16(v.w));
+          if (p.prep_m_prev) { v.x += x4[ps].x * mb; v.y += x4[ps].y * mb; v.z += x4[ps].z * mb; v.w += x4[ps].w * mb; }
+          *reinterpret_cast<float4*>(p.prep_d_out + e0 + ps * rstep) = v;
+          if (ext) *reinterpret_cast<float4*>(ext + ps * rstep) = v;
+          const float f0 = round_bf16(v.x), f1 = round_bf16(v.y), f2 = round_bf16(v.z), f3 = round_bf16(v.w);
+          Elem<uint16_t>::store4(p.prep_g16 + e0 + ps * rstep, f0, f1, f2, f3);
+          ss += f0 * f0 + f1 * f1 + f2 * f2 + f3 * f3;
+        }
+      }
+    }
+    ss = block_sum(ss, reinterpret_cast<float*>(smem));
+    if (threadIdx.x == 0) p.prep_ss_part[(size_t)bz * p.map.gy + tile] = ss;
+    return;
+  }
   float* out = p.add_out ? p.add_out + slot : p.partial + (size_t)split * p.map.gz * p.mat_elems + slot;
   const int r0 = ST::row0(), c0 = ST::col0();
   if (ST::active() && n0 + c0 < job.N) {

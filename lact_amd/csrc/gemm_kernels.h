@@ -346,6 +346,12 @@ struct TokenReduceParams {
   float* partial; long long mat_elems;
   // single split only (asynchronous-copy kernel): out = coeff*add_in + result written here instead of a partial
   float* add_out; const float* add_in; float coeff;
+  // single split only, forward update: what k_momentum_prep would do with the result, done by the epilogue --
+  // d_out = round_bf16(result) + m_prev * mbar[batch] (fp32 momentum state), its bf16 copy g16 in the same
+  // layout, and the sum of squares of that copy per block in ss_part[matrix][tile]
+  float* prep_d_out; const float* prep_m_prev; const float* prep_mbar; uint16_t* prep_g16; float* prep_ss_part;
+  float* prep_m_ext[3];    // caller's momentum outputs [b][elems] per matrix kind (same values as d_out), each nullable
+  ClearWords prep_clear;   // barrier lines of the fused Newton-Schulz kernel that follows (cleared by the first block)
 };
 
 template <typename T, class TS>

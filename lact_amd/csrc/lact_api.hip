@@ -626,8 +626,15 @@ struct Runner {
   // buffer (the caller reduces them), or 0 when the result went straight to `add_out` = coeff*add_in + sum.
   // bf16: whole blocks of 64 tokens run on the asynchronous-copy kernel (straight to add_out when one split
   // covers them); a ragged tail of fewer than 64 tokens goes through the generic kernel and is added.
+  // `prep` (forward update only): d_out / g16 / ss_part / m_prev / mbar of the momentum step; when the whole
+  // reduction is one split of the asynchronous-copy kernel, its epilogue does that step and -1 is returned.
+  struct PrepFold {
+    float* d_out; const float* m_prev; const float* mbar; uint16_t* g16; float* ss_part;
+    float* m_ext[3];
+    ClearWords clear;
+  };
   int token_reduce(const char* site, const TokenReduceJob (&jobs)[3], int tokens, float* add_out = nullptr,
-                   const float* add_in = nullptr, float coeff = 0.f) const {
+                   const float* add_in = nullptr, float coeff = 0.f, const PrepFold* prep = nullptr) const {
     TokenReduceParams p;
     memset(&p, 0, sizeof(p));
     for (int i = 0; i < 3; ++i) p.job[i] = jobs[i];
@@ -649,7 +656,12 @@ struct Runner {
         dim3 g(pd.map.grid());
         const double fl = 6.0 * main_tokens * d.d * d.dh * d.b * jobs[0].nterms;
         direct = add_out && sp.n == 1;
-        if (direct) { pd.add_out = add_out; pd.add_in = coeff != 0.f ? add_in : nullptr; pd.coeff = coeff; }
+        const bool folded = prep && sp.n == 1 && main_tokens == tokens;
+        if (folded) {
+          pd.prep_d_out = prep->d_out; pd.prep_m_prev = prep->m_prev; pd.prep_mbar = prep->mbar;
+          pd.prep_g16 = prep->g16; pd.prep_ss_part = prep->ss_part; pd.prep_clear = prep->clear;
+          for (int j = 0; j < 3; ++j) pd.prep_m_ext[j] = prep->m_ext[j];
+        } else if (direct) { pd.add_out = add_out; pd.add_in = coeff != 0.f ? add_in : nullptr; pd.coeff = coeff; }
         else slots = sp.n;
         if (big) {
           constexpr int SM = cmax(DmaSmem<TS_NS, 1, row_stages<TS_NS>()>::BYTES, StageTile<TS_NS, 4>::BYTES);
@@ -660,6 +672,7 @@ struct Runner {
           LACT_BIG_LDS(k_token_reduce_dma<TS_SQ>, SM);
           LACT_LAUNCH_SMEM("k_token_reduce_dma<128x128>", site, fl, (k_token_reduce_dma<TS_SQ>), g, dim3(DMA_THREADS), SM, s, pd);
         }
+        if (folded) return -1;
         if (main_tokens == tokens) return slots;
       }
     }
@@ -765,6 +778,8 @@ struct Runner {
         launch_hidden(1, hp, ver, T_);
         upd_z[0] = z0; upd_z[1] = z1; upd_z[2] = z2; upd_zbs = zbs;
       }
+      // mean of the momentum over the chunk (weighs the earlier state; the first update has none: never used)
+      if (P.momentum && u > 0) LACT_LAUNCH("k_momentum_mean", "k_momentum_mean", 0.0, k_momentum_mean, dim3(d.b), dim3(256), s, mom, (long long)d.kv_len, st.start, T_, mbar(u));
       int dw_slots = 0;
       {
         TokenReduceJob jobs[3];
@@ -776,11 +791,23 @@ struct Runner {
         set_tr_term(jobs[1].t[0], vc, d.v_ld, d.v_bs, upd_z[1], d.dh, upd_zbs);
         jobs[2].M = d.dh; jobs[2].N = d.d;
         set_tr_term(jobs[2].t[0], upd_z[2], d.dh, upd_zbs, kc, d.k_ld, d.k_bs);
-        dw_slots = token_reduce("update_dw", jobs, T_);
+        // square shapes with Muon: the momentum step can ride in the reduction's epilogue (every tile exists for
+        // every matrix, and the Newton-Schulz orientation is the packed one)
+        PrepFold pf;
+        const bool can_fold = kBf16 && kNsBf16 && P.muon && !P.g.stacked && d.d == d.dh;
+        if (can_fold) {
+          for (int j = 0; j < 3; ++j) pf.m_ext[j] = (u + 1 == P.nupd && P.momentum && m_out) ? m_out[j] : nullptr;
+          pf.d_out = dsave(u); pf.m_prev = (P.momentum && u > 0) ? dsave(u - 1) : nullptr;
+          pf.mbar = (P.momentum && u > 0) ? mbar(u) : nullptr;
+          pf.g16 = reinterpret_cast<uint16_t*>(g16(u)); pf.ss_part = scr<float>(P.t_ss);
+          pf.clear.ptr = nullptr; pf.clear.n = 0;
+          if (ns_all_fused()) pf.clear = ns_clear();
+        }
+        dw_slots = token_reduce("update_dw", jobs, T_, nullptr, nullptr, 0.f, can_fold ? &pf : nullptr);
       }
-      // the first update has no earlier momentum state to weigh: its mean is never used
-      if (P.momentum && u > 0) LACT_LAUNCH("k_momentum_mean", "k_momentum_mean", 0.0, k_momentum_mean, dim3(d.b), dim3(256), s, mom, (long long)d.kv_len, st.start, T_, mbar(u));
-      {
+      const bool prep_folded = dw_slots < 0;
+      const int ss_parts = prep_folded ? token_reduce_dma_tiles(d.d, d.dh) : P.nblk;
+      if (!prep_folded) {
         MomentumPrepParams p;
         memset(&p, 0, sizeof(p));
         p.g = P.g; p.partial = scr<float>(P.t_partial); p.nsplit = dw_slots;
@@ -801,7 +828,7 @@ struct Runner {
         if (!scale_in_kernel) {
           NsScaleParams p;
           memset(&p, 0, sizeof(p));
-          p.g = P.g; p.g16 = g16(u); p.ss_part = scr<float>(P.t_ss); p.nparts = P.nblk; p.norms = norms(u);
+          p.g = P.g; p.g16 = g16(u); p.ss_part = scr<float>(P.t_ss); p.nparts = ss_parts; p.norms = norms(u);
           p.xf = scr<float>(P.t_xf[0]); p.xb = xb(u, 0);
           p.u = P.S == 0 ? usave(u) : nullptr;
           p.plain_bf16 = d.ns_mode == LACT_NS_PLAIN_BF16;
@@ -820,7 +847,7 @@ struct Runner {
               f.xb_last = scr<uint16_t>(P.t_xbtmp) + B.xoff; f.u_out = usave(u) + B.xoff;
               if (scale_in_kernel) {
                 f.g16 = reinterpret_cast<const uint16_t*>(g16(u)) + B.xoff;
-                f.ss_part = scr<float>(P.t_ss); f.nparts = P.nblk;
+                f.ss_part = scr<float>(P.t_ss); f.nparts = ss_parts;
                 f.part0 = B.first; f.part1 = (P.g.stacked && B.first == 0) ? 2 * d.b : -1;
                 f.norms = norms(u) + B.first;
               }

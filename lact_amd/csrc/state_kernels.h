@@ -95,16 +95,6 @@ __global__ void k_init_state(const InitParams p) {
   if (lane == 0) p.n0[(size_t)z * p.g.maxrows() + row] = sqrtf(ss);
 }
 
-// Side job of a kernel that runs right before a fused Newton-Schulz launch: its first block clears the barrier
-// lines and the error word (a few KiB), which saves a launch of its own in the dependent chain.
-struct ClearWords {
-  unsigned* ptr; int n;
-};
-__device__ __forceinline__ void clear_words(const ClearWords& c, bool first_block) {
-  if (c.n > 0 && first_block)
-    for (int i = threadIdx.x; i < c.n; i += blockDim.x) c.ptr[i] = 0u;
-}
-
 // ---- mean of the per-token momentum over one chunk (ttt_operation.py:171-172) --------------------
 __global__ void k_momentum_mean(const float* mom, long long bs, int start, int len, float* mbar) {
   __shared__ float red[16];
