@@ -70,6 +70,9 @@ typedef struct lact_desc {
   /* No lact_backward call follows (inference, torch.no_grad): the forward keeps no activations for it, `saved` is
    * smaller, and lact_backward refuses the descriptor.  No counterpart in the reference, where autograd decides. */
   int32_t forward_only;
+  /* The first update starts from a momentum state carried in by the caller (lact_forward_from_state) instead of
+   * zero: ar_lact_swa_repeat_sp.py:215-217,266-269,309-317.  Needs use_momentum and forward_only. */
+  int32_t momentum_state_in;
 } lact_desc_t;
 
 const char* lact_last_error(void);
@@ -90,6 +93,15 @@ int lact_forward(const lact_desc_t* desc, const float* w0, const float* w1, cons
                  const void* k, const void* v, const float* lr0, const float* lr1, const float* lr2,
                  const float* momentum, void* out, float* const w_out[3], float* const m_out[3], void* saved,
                  void* scratch, void* stream);
+
+/* lact_forward with the momentum states of an earlier call carried in: m_in[3] (fp32, shapes of w0,w1,w2) is what
+ * that call returned through m_out.  Replaces ar_fast_weight_swish_glu_weight_norm_mini_batch_inference_with_momentum
+ * (ar_lact_swa_repeat_sp.py:197-339), whose caller keeps the states between denoising steps (:998-1053).
+ * desc->momentum_state_in must be set (and m_in null when it is not); inference only. */
+int lact_forward_from_state(const lact_desc_t* desc, const float* w0, const float* w1, const float* w2, const void* q,
+                            const void* k, const void* v, const float* lr0, const float* lr1, const float* lr2,
+                            const float* momentum, const float* const m_in[3], void* out, float* const w_out[3],
+                            float* const m_out[3], void* saved, void* scratch, void* stream);
 
 /* Backward of the same program (the reference relies on autograd; closed forms as in
  * lact_triton_kernels/lact_swiglu_ffn.py:46-76, lact_fw_grad.py:61-156, l2norm_triton_kernels.py:106-172).

@@ -30,11 +30,12 @@ class Desc(Structure):
         ("q_bs", c_int64), ("k_bs", c_int64), ("v_bs", c_int64), ("o_bs", c_int64), ("do_bs", c_int64),
         ("q_ld", c_int32), ("k_ld", c_int32), ("v_ld", c_int32), ("o_ld", c_int32), ("do_ld", c_int32),
         ("muon_stacked", c_int32), ("renorm_eps_in_sqrt", c_int32), ("forward_only", c_int32),
+        ("momentum_state_in", c_int32),
     ]
 
 
 OPT_STREAM_OVERLAP, OPT_FUSED_NEWTON_SCHULZ = 0, 1
-EXPORTS = ("lact_last_error", "lact_version", "lact_query_sizes", "lact_forward", "lact_backward",
+EXPORTS = ("lact_last_error", "lact_version", "lact_query_sizes", "lact_forward", "lact_forward_from_state", "lact_backward",
            "lact_newton_schulz_workspace_bytes", "lact_newton_schulz", "lact_set_option", "lact_profile_enable",
            "lact_profile_report", "lact_layer_pre_forward", "lact_layer_pre_backward", "lact_layer_lr_forward",
            "lact_layer_lr_backward", "lact_layer_post_forward", "lact_layer_post_dw_rows", "lact_layer_post_backward")
@@ -58,6 +59,8 @@ def lib():
     vp = c_void_p
     L.lact_forward.argtypes = [POINTER(Desc)] + [vp] * 10 + [vp, POINTER(vp), POINTER(vp), vp, vp, vp]
     L.lact_forward.restype = c_int32
+    L.lact_forward_from_state.argtypes = [POINTER(Desc)] + [vp] * 10 + [POINTER(vp), vp, POINTER(vp), POINTER(vp), vp, vp, vp]
+    L.lact_forward_from_state.restype = c_int32
     L.lact_backward.argtypes = [POINTER(Desc)] + [vp] * 8 + [POINTER(vp), vp, vp] + [vp] * 10 + [vp]
     L.lact_backward.restype = c_int32
     L.lact_newton_schulz_workspace_bytes.argtypes = [c_int32] * 4

@@ -196,10 +196,10 @@ struct Plan {
   std::vector<float> coeffs;
   MatGeom g;
   int nupd = 0, Tcap = 0, S = -1, esz = 2, nsz = 2, r = 0, c = 0, nblk = 1, lr_slots = 1, tiles = 1, nsplit_max = 1;
-  bool muon = false, bf16 = true, momentum = false;
+  bool muon = false, bf16 = true, momentum = false, state_in = false;
   size_t mat3 = 0;  // 3*b*elems
   // saved
-  size_t s_n0, s_wf, s_wc, s_main, s_d, s_mbar, s_u, s_g16, s_norms, s_xb, s_ab, s_bb, saved_bytes;
+  size_t s_n0, s_wf, s_wc, s_main, s_d, s_min, s_mbar, s_u, s_g16, s_norms, s_xb, s_ab, s_bb, saved_bytes;
   // Kept for the backward on the asynchronous-copy path: per update, six token-major arrays [b][T][dh] -- the three
   // lr-scaled operands of the fast-weight gradient GEMMs and the three rounded pre-activations they came from.
   // 288 GB of HBM make keeping them cheaper than the three GEMMs that would recompute them.
@@ -232,6 +232,9 @@ struct Plan {
     if (S > 64) return fail("too many Newton-Schulz steps");
     if (S > 0) coeffs.assign(d.ns_coeffs, d.ns_coeffs + 3 * S);
     momentum = d.use_momentum != 0;
+    state_in = d.momentum_state_in != 0;
+    if (state_in && (!momentum || !d.forward_only))
+      return fail("momentum_state_in needs use_momentum and forward_only (the carried state has no backward pass)");
     if (d.ns_mode < 0 || d.ns_mode > 2) return fail("ns_mode must be 0, 1 or 2");
     nsz = d.ns_mode == LACT_NS_FP32 ? 4 : 2;
     nupd = 0;
@@ -281,6 +284,7 @@ struct Plan {
     s_wc = bf16 ? sv.take((size_t)(nupd + 1) * mat3 * 2) : s_wf;
     s_main = d.prenorm ? sv.take((size_t)nupd * mat3 * 4) : 0;
     s_d = sv.take((size_t)nupd * mat3 * 4);
+    s_min = state_in ? sv.take(mat3 * 4) : 0;
     s_mbar = sv.take((size_t)std::max(1, nupd) * d.b * 4);
     s_u = muon ? sv.take((size_t)nupd * mat3 * 4) : 0;
     s_g16 = muon ? sv.take((size_t)nupd * mat3 * nsz) : 0;
@@ -551,6 +555,9 @@ struct Runner {
   // accumulator after `u` updates (pre-norm); main(0) is the initial weight
   float* main_(int u) const { return u == 0 ? wf(0) : reinterpret_cast<float*>(sv + P.s_main) + (size_t)(u - 1) * P.mat3; }
   float* dsave(int u) const { return reinterpret_cast<float*>(sv + P.s_d) + (size_t)u * P.mat3; }
+  // momentum state that update `u` starts from: the previous update's, or the one the caller carried in
+  bool has_prev(int u) const { return P.momentum && (u > 0 || P.state_in); }
+  const float* mprev(int u) const { return !has_prev(u) ? nullptr : u > 0 ? dsave(u - 1) : reinterpret_cast<const float*>(sv + P.s_min); }
   float* mbar(int u) const { return reinterpret_cast<float*>(sv + P.s_mbar) + (size_t)u * d.b; }
   float* usave(int u) const { return reinterpret_cast<float*>(sv + P.s_u) + (size_t)u * P.mat3; }
   TN* g16(int u) const { return reinterpret_cast<TN*>(sv + P.s_g16) + (size_t)u * P.mat3; }
@@ -715,8 +722,15 @@ struct Runner {
 
   // ------------------------------------------------------------------------------------------
   int forward(const float* w0, const float* w1, const float* w2, const T* q, const T* k, const T* v, const float* lr0,
-              const float* lr1, const float* lr2, const float* mom, T* out, float* const w_out[3], float* const m_out[3]) {
+              const float* lr1, const float* lr2, const float* mom, T* out, float* const w_out[3], float* const m_out[3],
+              const float* const m_in[3]) {
     const dim3 rowgrid(ceil_div(P.g.maxrows(), 4), 3 * d.b);
+    // carried momentum state: packed like every other state array (a device-to-device copy node when captured)
+    if (P.state_in && P.nupd > 0)
+      for (int j = 0; j < 3; ++j)
+        if (hipMemcpyAsync(sv + P.s_min + (size_t)j * d.b * P.g.elems * 4, m_in[j], (size_t)d.b * P.g.elems * 4,
+                           hipMemcpyDeviceToDevice, s) != hipSuccess)
+          return fail("copy of the carried momentum state failed");
     {
       InitParams p;
       p.g = P.g; p.w[0] = w0; p.w[1] = w1; p.w[2] = w2; p.n0 = n0(); p.wf = wf(0);
@@ -779,7 +793,7 @@ struct Runner {
         upd_z[0] = z0; upd_z[1] = z1; upd_z[2] = z2; upd_zbs = zbs;
       }
       // mean of the momentum over the chunk (weighs the earlier state; the first update has none: never used)
-      if (P.momentum && u > 0) LACT_LAUNCH("k_momentum_mean", "k_momentum_mean", 0.0, k_momentum_mean, dim3(d.b), dim3(256), s, mom, (long long)d.kv_len, st.start, T_, mbar(u));
+      if (has_prev(u)) LACT_LAUNCH("k_momentum_mean", "k_momentum_mean", 0.0, k_momentum_mean, dim3(d.b), dim3(256), s, mom, (long long)d.kv_len, st.start, T_, mbar(u));
       int dw_slots = 0;
       {
         TokenReduceJob jobs[3];
@@ -797,8 +811,8 @@ struct Runner {
         const bool can_fold = kBf16 && kNsBf16 && P.muon && !P.g.stacked && d.d == d.dh;
         if (can_fold) {
           for (int j = 0; j < 3; ++j) pf.m_ext[j] = (u + 1 == P.nupd && P.momentum && m_out) ? m_out[j] : nullptr;
-          pf.d_out = dsave(u); pf.m_prev = (P.momentum && u > 0) ? dsave(u - 1) : nullptr;
-          pf.mbar = (P.momentum && u > 0) ? mbar(u) : nullptr;
+          pf.d_out = dsave(u); pf.m_prev = mprev(u);
+          pf.mbar = has_prev(u) ? mbar(u) : nullptr;
           pf.g16 = reinterpret_cast<uint16_t*>(g16(u)); pf.ss_part = scr<float>(P.t_ss);
           pf.clear.ptr = nullptr; pf.clear.n = 0;
           if (ns_all_fused()) pf.clear = ns_clear();
@@ -811,8 +825,8 @@ struct Runner {
         MomentumPrepParams p;
         memset(&p, 0, sizeof(p));
         p.g = P.g; p.partial = scr<float>(P.t_partial); p.nsplit = dw_slots;
-        p.m_prev = (P.momentum && u > 0) ? dsave(u - 1) : nullptr;
-        p.mbar = (P.momentum && u > 0) ? mbar(u) : nullptr;
+        p.m_prev = mprev(u);
+        p.mbar = has_prev(u) ? mbar(u) : nullptr;
         p.d_out = dsave(u);
         p.g16 = P.muon ? g16(u) : nullptr;
         p.ss_part = scr<float>(P.t_ss);
@@ -1571,8 +1585,18 @@ int lact_query_sizes(const lact_desc_t* desc, size_t* saved_bytes, size_t* scrat
 int lact_forward(const lact_desc_t* desc, const float* w0, const float* w1, const float* w2, const void* q, const void* k,
                  const void* v, const float* lr0, const float* lr1, const float* lr2, const float* momentum, void* out,
                  float* const w_out[3], float* const m_out[3], void* saved, void* scratch, void* stream) {
+  return lact_forward_from_state(desc, w0, w1, w2, q, k, v, lr0, lr1, lr2, momentum, nullptr, out, w_out, m_out, saved,
+                                 scratch, stream);
+}
+
+int lact_forward_from_state(const lact_desc_t* desc, const float* w0, const float* w1, const float* w2, const void* q,
+                            const void* k, const void* v, const float* lr0, const float* lr1, const float* lr2,
+                            const float* momentum, const float* const m_in[3], void* out, float* const w_out[3],
+                            float* const m_out[3], void* saved, void* scratch, void* stream) {
   Plan P;
   if (P.build(desc)) return -1;
+  if (P.state_in && (!m_in || !m_in[0] || !m_in[1] || !m_in[2])) return fail("momentum_state_in set but a state pointer is null");
+  if (!P.state_in && m_in) return fail("momentum state passed without momentum_state_in in the descriptor");
   if (check_ptrs({w0, w1, w2, q, out, saved, scratch}, "forward tensors")) return -1;
   if (P.nupd > 0 && check_ptrs({k, v, lr0, lr1, lr2}, "k, v, lr")) return -1;
   if (P.nupd > 0 && P.momentum && !momentum) return fail("use_momentum set but momentum is null");
@@ -1582,7 +1606,7 @@ int lact_forward(const lact_desc_t* desc, const float* w0, const float* w1, cons
   {                                                                                                                 \
     Runner<T_, TN_> R(P, saved, scratch, s);                                                                        \
     return R.forward(w0, w1, w2, (const T_*)q, (const T_*)k, (const T_*)v, lr0, lr1, lr2, momentum, (T_*)out, w_out, \
-                     m_out);                                                                                        \
+                     m_out, m_in);                                                                                  \
   }
   const bool ns32 = P.d.ns_mode == LACT_NS_FP32;
   if (P.bf16 && !ns32) LACT_FWD(uint16_t, uint16_t)

@@ -141,7 +141,7 @@ def _covers(steps, out_len: int) -> bool:
 
 class _LactProgramFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, prog: Program, w0, w1, w2, q, k, v, lr0, lr1, lr2, momentum):
+    def forward(ctx, prog: Program, w0, w1, w2, q, k, v, lr0, lr1, lr2, momentum, m_state=None):
         if not q.is_cuda:
             raise RuntimeError("lact_amd runs on an MI355X only: tensors must be on a HIP device (no CPU path)")
         L = _lib.lib()
@@ -164,6 +164,14 @@ class _LactProgramFn(torch.autograd.Function):
         call = _Call(prog, b, d, dh, qa, ka, va, out)
         call.desc.use_momentum = int(mom is not None)
         call.desc.forward_only = int(not any(ctx.needs_input_grad))
+        m_in = None
+        if m_state is not None and mom is not None:
+            if not call.desc.forward_only:
+                raise RuntimeError("a carried momentum state is an inference feature: call under torch.no_grad()")
+            m_in = [m.detach().float().contiguous() for m in m_state]
+            if any(m.shape != w.shape for m, w in zip(m_in, wf)):
+                raise ValueError("momentum states must have the shapes of w0, w1, w2")
+            call.desc.momentum_state_in = 1
         saved_bytes, scratch_bytes = call.sizes()
         saved = torch.empty(saved_bytes, dtype=torch.uint8, device=q.device)
         scratch = torch.empty(scratch_bytes, dtype=torch.uint8, device=q.device)
@@ -171,9 +179,10 @@ class _LactProgramFn(torch.autograd.Function):
         m_out = [torch.empty_like(w) for w in wf] if (mom is not None and prog.return_state) else [None, None, None]
         stream = ctypes.c_void_p(torch.cuda.current_stream(q.device).cuda_stream)
         with torch.cuda.device(q.device):
-            _lib.check(L.lact_forward(ctypes.byref(call.desc), _ptr(wf[0]), _ptr(wf[1]), _ptr(wf[2]), _ptr(qa), _ptr(ka),
-                                      _ptr(va), _ptr(lrs[0]), _ptr(lrs[1]), _ptr(lrs[2]), _ptr(mom), _ptr(out),
-                                      _ptr3(w_out), _ptr3(m_out), _ptr(saved), _ptr(scratch), stream))
+            _lib.check(L.lact_forward_from_state(
+                ctypes.byref(call.desc), _ptr(wf[0]), _ptr(wf[1]), _ptr(wf[2]), _ptr(qa), _ptr(ka), _ptr(va), _ptr(lrs[0]),
+                _ptr(lrs[1]), _ptr(lrs[2]), _ptr(mom), None if m_in is None else _ptr3(m_in), _ptr(out), _ptr3(w_out),
+                _ptr3(m_out), _ptr(saved), _ptr(scratch), stream))
         ctx.prog, ctx.dims = prog, (b, d, dh)
         ctx.in_dtypes = (w0.dtype, w1.dtype, w2.dtype, q.dtype, k.dtype if k is not None else None,
                          v.dtype if v is not None else None)
@@ -231,13 +240,14 @@ class _LactProgramFn(torch.autograd.Function):
         glr = [None if g is None else g.reshape(lr_shape).to(ctx.lr_dtype) for g in dlr]
         gm = None if dmom is None else dmom.reshape(mom_shape).to(ctx.mom_dtype)
         return (None, cast(dw[0], wd0), cast(dw[1], wd1), cast(dw[2], wd2), cast(dq, qd), cast(dk, kd), cast(dv, vd),
-                glr[0], glr[1], glr[2], gm)
+                glr[0], glr[1], glr[2], gm, None)
 
 
 @torch.compiler.disable
-def run_program(prog: Program, w0, w1, w2, q, k, v, lr0, lr1, lr2, momentum=None):
-    """Runs `prog`.  Returns (out, (w0, w1, w2) after the last update, (m0, m1, m2) momentum states)."""
-    res = _LactProgramFn.apply(prog, w0, w1, w2, q, k, v, lr0, lr1, lr2, momentum)
+def run_program(prog: Program, w0, w1, w2, q, k, v, lr0, lr1, lr2, momentum=None, momentum_state=None):
+    """Runs `prog`.  Returns (out, (w0, w1, w2) after the last update, (m0, m1, m2) momentum states).
+    `momentum_state` = the (m0, m1, m2) of an earlier call: the first update continues from it (inference only)."""
+    res = _LactProgramFn.apply(prog, w0, w1, w2, q, k, v, lr0, lr1, lr2, momentum, momentum_state)
     return res[0], res[1:4], res[4:7]
 
 

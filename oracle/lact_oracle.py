@@ -196,7 +196,8 @@ def run_program(w0, w1, w2, q, k, v, lr0, lr1, lr2, steps: Sequence[Step], *,
                 out_rows: Optional[int] = None,
                 scatter_output: bool = True,
                 stack_muon: bool = False,
-                eps_in_sqrt: bool = False):
+                eps_in_sqrt: bool = False,
+                momentum_state: Optional[Sequence[torch.Tensor]] = None):
     """Runs UPDATE / APPLY steps over one sequence.  LLM layout: w0,w2 [b,dh,dk], w1 [b,dv,dh].
 
     ns_coeffs=None means no Muon.  `muon_replaces_weight` is the bidirectional layer's behaviour
@@ -215,6 +216,8 @@ def run_program(w0, w1, w2, q, k, v, lr0, lr1, lr2, steps: Sequence[Step], *,
     mom = None
     if momentum is not None:                        # ttt_operation.py:112-115
         mom = [torch.zeros_like(w0), torch.zeros_like(w1), torch.zeros_like(w2)]
+        if momentum_state is not None:              # ar_lact_swa_repeat_sp.py:266-269 (state carried between calls)
+            mom = list(momentum_state)
 
     pieces: List[Tuple[int, int, torch.Tensor]] = []
     for kind, s, e in steps:
@@ -425,6 +428,31 @@ def ar_fast_weight_swish_glu_weight_norm_mini_batch_inference(w0, w1, w2, q, k, 
         ns_coeffs=ns_coeff_table("classic", num_moun_iters) if use_moun else None,
         weight_norm=weight_norm, cast_lr_operand=False)
     return (out,) + tuple(ws)
+
+
+def ar_fast_weight_swish_glu_weight_norm_mini_batch_inference_with_momentum(
+        w0, w1, w2, q, k, v, lr0, lr1, lr2, w_scale: float, num_repeat: int = 1, mini_batch_size: int = -1,
+        do_update: bool = False, use_moun: bool = False, num_moun_iters: int = 3, weight_norm: bool = True,
+        fw_momentum: Optional[torch.Tensor] = None, dw0_momentum=None, dw1_momentum=None, dw2_momentum=None,
+        use_momentum: bool = False, *, num: Numerics = Numerics()):
+    """ar_lact_swa_repeat_sp.py:197-339: the inference step whose momentum states travel between calls.
+    Returns (output, w0, w1, w2, m0, m1, m2); the states come back untouched when no update runs, as zeros when
+    momentum is on and none were given (:266-269), and as None when momentum is off."""
+    mb = k.shape[1] if mini_batch_size == -1 else mini_batch_size
+    steps = [Step(UPDATE, 0, mb) for _ in range(num_repeat)] if do_update else []
+    steps.append(Step(APPLY, 0, q.shape[1]))
+    state = None
+    if use_momentum:
+        state = ((dw0_momentum, dw1_momentum, dw2_momentum) if dw0_momentum is not None
+                 else (torch.zeros_like(w0), torch.zeros_like(w1), torch.zeros_like(w2)))
+    out, ws, ms = run_program(
+        w0, w1, w2, q, k, v, lr0 * w_scale, lr1 * w_scale, lr2 * w_scale, steps, num=num,
+        ns_coeffs=ns_coeff_table("classic", num_moun_iters) if use_moun else None,
+        momentum=fw_momentum if use_momentum else None, weight_norm=weight_norm,
+        cast_lr_operand=False, momentum_state=state)
+    if not use_momentum:
+        ms = (dw0_momentum, dw1_momentum, dw2_momentum)
+    return (out,) + tuple(ws) + tuple(ms)
 
 
 # ---------------------------------------------------------------------------------------------

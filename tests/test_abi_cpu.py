@@ -84,6 +84,13 @@ def test_query_sizes_and_validation_messages():
     fo = make_desc(ops.block_causal_steps(256, 64), forward_only=1)
     assert L.lact_backward(ctypes.byref(fo), *([null] * 22)) != 0
     assert "forward_only" in L.lact_last_error().decode()
+    # a carried momentum state is an inference feature: needs use_momentum and forward_only, and costs one more
+    # state array in `saved`
+    assert "momentum_state_in" in err(make_desc(ops.block_causal_steps(256, 64), momentum_state_in=1, use_momentum=1))
+    assert "momentum_state_in" in err(make_desc(ops.block_causal_steps(256, 64), momentum_state_in=1, forward_only=1))
+    rc, saved_mo, _ = sizes(make_desc(ops.block_causal_steps(256, 64), forward_only=1, use_momentum=1))
+    rc2, saved_st, _ = sizes(make_desc(ops.block_causal_steps(256, 64), forward_only=1, use_momentum=1, momentum_state_in=1))
+    assert rc == 0 and rc2 == 0 and saved_st > saved_mo
     assert L.lact_query_sizes(None, None, None) != 0 and "null" in L.lact_last_error().decode()
     assert L.lact_newton_schulz_workspace_bytes(4, 64, 128, 5) > 0
     assert L.lact_newton_schulz_workspace_bytes(0, 64, 128, 5) == 0

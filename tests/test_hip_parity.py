@@ -408,6 +408,116 @@ def test_ar_video_inference_repeat_accumulates_kv_grads():
     assert max(errs.values()) < 1e-4
 
 
+INF_M = ar_video.ar_fast_weight_swish_glu_weight_norm_mini_batch_inference_with_momentum
+INF_M_ORACLE = O.ar_fast_weight_swish_glu_weight_norm_mini_batch_inference_with_momentum
+
+
+@pytest.mark.parametrize("d,dh,act,use_moun,weight_norm,repeat", [
+    (64, 128, torch.float32, False, True, 1), (64, 128, torch.float32, False, False, 2),
+    (128, 128, torch.float32, True, True, 1),       # fp32 Newton-Schulz against float64 (exact arithmetic)
+    (64, 128, torch.bfloat16, False, True, 2), (128, 128, torch.bfloat16, True, True, 1),
+    (384, 384, torch.bfloat16, True, True, 2),      # fused Newton-Schulz, momentum step in the reduction's epilogue
+    (40, 136, torch.bfloat16, False, True, 1)])
+def test_ar_video_inference_with_carried_momentum_state(d, dh, act, use_moun, weight_norm, repeat):
+    """ar_lact_swa_repeat_sp.py:197-339: the first update continues from the states of an earlier call."""
+    say("ar video inference with momentum state", d, dh, act, use_moun, weight_norm, repeat)
+    b, L, mb = 3, 200, 128
+    inp = problem(b, L, d, dh, 21, act, momentum=True, lr_shift=-1.0)
+    gen = torch.Generator().manual_seed(77)
+    M = [0.02 * torch.randn(w.shape, generator=gen) for w in (inp["w0"], inp["w1"], inp["w2"])]
+    exact = use_moun and act == torch.float32
+    num = EXACT if exact else (AC if act == torch.bfloat16 else PLAIN)
+    cast = (lambda t: t.double()) if exact else (lambda t: t)
+    c = {n: (None if t is None else cast(t)) for n, t in inp.items()}
+    with torch.no_grad():
+        ref = INF_M_ORACLE(*args9(c), 0.5, repeat, mb, True, use_moun, 3, weight_norm, c["momentum"],
+                           cast(M[0]), cast(M[1]), cast(M[2]), True, num=num)
+        g = clone_to(inp, DEV, grad=False)
+        Mg = [m.to(DEV) for m in M]
+        run = lambda: INF_M(*args9(g), 0.5, repeat, mb, True, use_moun, 3, weight_norm, g["momentum"], Mg[0], Mg[1],
+                            Mg[2], True)
+        if exact:
+            with ops.newton_schulz_mode(ops.NS_FP32):
+                res = run()
+        else:
+            res = run()
+        torch.cuda.synchronize()
+        names = ["out", "w0", "w1", "w2", "m0", "m1", "m2"]
+        errs = {n: O.rel_l2(r, f) for n, r, f in zip(names, res, ref)}
+        say("  ", errs)
+        if use_moun and not exact:
+            # bf16 Newton-Schulz: bounded by the oracle's own distance from float64 arithmetic
+            c64 = {n: (None if t is None else t.double()) for n, t in inp.items()}
+            r64 = INF_M_ORACLE(*args9(c64), 0.5, repeat, mb, True, use_moun, 3, weight_norm, c64["momentum"],
+                               M[0].double(), M[1].double(), M[2].double(), True, num=EXACT)
+            for n, r, f, x in zip(names, res, ref, r64):
+                floor = O.rel_l2(f, x)
+                assert O.rel_l2(r, x) <= 1.25 * floor + 2e-3 and O.rel_l2(r, f) <= 2.0 * floor + 2e-3, n
+        else:
+            tol = 1e-3 if exact else (1e-2 if act == torch.bfloat16 else 1e-4)
+            assert max(errs.values()) < tol
+        # without a state the same call differs (the state is really used)
+        bare = INF_M(*args9(g), 0.5, repeat, mb, True, use_moun, 3, weight_norm, g["momentum"], None, None, None, True)
+        assert O.rel_l2(bare[4], res[4]) > 1e-2
+
+
+def test_carried_momentum_state_equals_one_longer_program_bitwise():
+    """Two calls that hand weights and states over do the arithmetic of one call with two updates (no weight norm,
+    so nothing is re-derived from the handed-over weights): same kernels, same bits."""
+    say("carried state: two calls against one")
+    inp = problem(2, 160, 64, 128, 22, torch.float32, momentum=True, lr_shift=-1.0)
+    with torch.no_grad():
+        g = clone_to(inp, DEV, grad=False)
+        both = INF_M(*args9(g), 0.7, 2, 96, True, False, 3, False, g["momentum"], None, None, None, True)
+        one = INF_M(*args9(g), 0.7, 1, 96, True, False, 3, False, g["momentum"], None, None, None, True)
+        two = INF_M(one[1], one[2], one[3], g["q"], g["k"], g["v"], g["lr0"], g["lr1"], g["lr2"], 0.7, 1, 96, True, False,
+                    3, False, g["momentum"], one[4], one[5], one[6], True)
+        torch.cuda.synchronize()
+        for n, a, b_ in zip(["out", "w0", "w1", "w2", "m0", "m1", "m2"], both, two):
+            assert torch.equal(a, b_), n
+        # no update: states and weights pass through, momentum off: states handed back as given
+        idle = INF_M(*args9(g), 0.7, 1, 96, False, False, 3, True, g["momentum"], one[4], one[5], one[6], True)
+        assert idle[4] is one[4] and torch.equal(idle[1], g["w0"])
+        off = INF_M(*args9(g), 0.7, 1, 96, True, False, 3, True, None, None, None, None, False)
+        assert off[4] is None
+    # a carried state has no backward pass: refused when a gradient is wanted
+    gg = clone_to(inp, DEV)
+    with pytest.raises(RuntimeError, match="inference"):
+        INF_M(*args9(gg), 0.7, 1, 96, True, False, 3, True, gg["momentum"], one[4], one[5], one[6], True)
+
+
+def test_fast_weight_inference_cache_follows_the_layer_protocol():
+    """ar_lact_swa_repeat_sp.py:998-1053,1147-1148: conditional and guidance sequences alternate, each with its own
+    weights and momentum states; both restart from the layer's parameters until each has been updated once."""
+    say("fast-weight inference cache")
+    b, L, d, dh = 2, 96, 64, 64
+    base = problem(b, L, d, dh, 23, torch.float32, momentum=True, lr_shift=-1.0)
+    chunks = [problem(b, L, d, dh, 30 + i, torch.float32, momentum=True, lr_shift=-1.0) for i in range(6)]
+    do_update = [True, True, False, False, True, True]
+    cache = ar_video.FastWeightInferenceCache(use_momentum=True)
+    held = {False: None, True: None}      # the oracle's copy of the protocol, written out call by call
+    cfg = False
+    with torch.no_grad():
+        W = [base[n].to(DEV) for n in ("w0", "w1", "w2")]
+        for i, (ch, upd) in enumerate(zip(chunks, do_update)):
+            g = clone_to(ch, DEV, grad=False)
+            out = cache.step(W[0], W[1], W[2], g["q"], g["k"], g["v"], g["lr0"], g["lr1"], g["lr2"], 0.5, do_update=upd,
+                             frames=3, fw_momentum=g["momentum"], mini_batch_size=64)
+            fresh = held[False] is None or held[True] is None
+            st = (base["w0"], base["w1"], base["w2"], None, None, None) if fresh else held[cfg]
+            ref = INF_M_ORACLE(st[0], st[1], st[2], ch["q"], ch["k"], ch["v"], ch["lr0"], ch["lr1"], ch["lr2"], 0.5, 1, 64,
+                               upd, False, 3, True, ch["momentum"], st[3], st[4], st[5], True, num=PLAIN)
+            if upd:
+                held[cfg] = tuple(ref[1:])
+            cfg = not cfg
+            e = O.rel_l2(out, ref[0])
+            say("   call", i, "update" if upd else "apply", "err", e)
+            assert e < 1e-4
+    assert cache.frame_offset == 6 and cache.cfg_seq is False      # two updating conditional calls, three frames each
+    cache.reset()
+    assert cache.cur is None and cache.frame_offset == 0
+
+
 # ---- size-independent properties at the benchmark size ----------------------------------------------
 def full_size_properties(b, L, d, dh, C, seed, single_update):
     inp = O.make_inputs(b, L, d, dh, seed=seed, act_dtype=torch.bfloat16, distinct_heads=4)

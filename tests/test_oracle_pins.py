@@ -347,3 +347,40 @@ def test_fused_variant_entry_points_share_schedule_and_differ_only_in_the_two_sw
     a = O.prenorm_block_causal_lact_swiglu_fused_kernel_triton(w0, w1, w2, q, k, v, lr0, lr1, lr2, 16, True, mom, num=F64)
     b_ = O.prenorm_block_causal_lact_swiglu(w0, w1, w2, q, k, v, lr0, lr1, lr2, 16, True, mom, num=F64)
     assert torch.equal(a[:, :16], b_[:, :16]) and O.rel_l2(a[:, 16:], b_[:, 16:]) > 1e-3
+
+
+# ---- inference step with momentum states carried between calls ------------------------------------------
+def test_carried_momentum_state_composes_and_is_the_heavy_ball_step():
+    """ar_lact_swa_repeat_sp.py:197-339.  (1) Without weight norm the states and weights after two calls, each
+    doing one update and handing its results to the next, equal one call doing both updates (a dropped or
+    re-zeroed state fails).  (2) A call with a given state M adds exactly mean(momentum) * M to the step a call
+    without state makes, on every weight, and returns step + that as the new state (wrong sign, wrong mean, a
+    state applied to the wrong weight fail).  (3) States pass through untouched when nothing updates."""
+    w0, w1, w2, q, k, v, lr0, lr1, lr2 = rand_problem(seed=5)
+    mom = torch.sigmoid(torch.randn(2, 40, 1, dtype=torch.float64))
+    fn = O.ar_fast_weight_swish_glu_weight_norm_mini_batch_inference_with_momentum
+    kw = dict(num=F64)
+    both = fn(w0, w1, w2, q, k, v, lr0, lr1, lr2, 0.7, 2, 24, True, False, 3, False, mom, None, None, None, True, **kw)
+    one = fn(w0, w1, w2, q, k, v, lr0, lr1, lr2, 0.7, 1, 24, True, False, 3, False, mom, None, None, None, True, **kw)
+    two = fn(one[1], one[2], one[3], q, k, v, lr0, lr1, lr2, 0.7, 1, 24, True, False, 3, False, mom, one[4], one[5],
+             one[6], True, **kw)
+    for a, b_ in zip(both, two):
+        assert torch.allclose(a, b_, atol=1e-12)
+    # (2): same weights, with and without a state
+    M = [torch.randn_like(w) for w in (w0, w1, w2)]
+    bare = fn(w0, w1, w2, q, k, v, lr0, lr1, lr2, 0.7, 1, 24, True, False, 3, False, mom, None, None, None, True, **kw)
+    with_m = fn(w0, w1, w2, q, k, v, lr0, lr1, lr2, 0.7, 1, 24, True, False, 3, False, mom, M[0], M[1], M[2], True, **kw)
+    mbar = mom[:, :24].mean(dim=1, keepdim=True)
+    for j, w in enumerate((w0, w1, w2)):
+        step = bare[1 + j] - w
+        assert torch.allclose(bare[4 + j], step, atol=1e-12)                     # first state = first step
+        assert torch.allclose(with_m[1 + j] - w, step + mbar * M[j], atol=1e-12)
+        assert torch.allclose(with_m[4 + j], step + mbar * M[j], atol=1e-12)
+    # (3)
+    idle = fn(w0, w1, w2, q, k, v, lr0, lr1, lr2, 0.7, 1, 24, False, False, 3, True, mom, M[0], M[1], M[2], True, **kw)
+    assert all(idle[4 + j] is M[j] for j in range(3)) and all(idle[1 + j] is w for j, w in enumerate((w0, w1, w2)))
+    assert torch.allclose(idle[0], O.swiglu_apply(w0, w1, w2, q, F64), atol=1e-12)
+    zeros = fn(w0, w1, w2, q, k, v, lr0, lr1, lr2, 0.7, 1, 24, False, False, 3, True, mom, None, None, None, True, **kw)
+    assert all(float(zeros[4 + j].abs().max()) == 0.0 for j in range(3))
+    off = fn(w0, w1, w2, q, k, v, lr0, lr1, lr2, 0.7, 1, 24, True, False, 3, True, None, None, None, None, False, **kw)
+    assert off[4] is None and off[5] is None and off[6] is None
