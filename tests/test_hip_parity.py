@@ -518,6 +518,45 @@ def test_fast_weight_inference_cache_follows_the_layer_protocol():
     assert cache.cur is None and cache.frame_offset == 0
 
 
+def test_video_model_shape_full_size_equals_its_inference_rollout():
+    """The video model's own shape (lact_ar_chunk3f_1.3B.yaml: 2 heads of 768, hidden 1536, 4680-token windows,
+    update_every 9360, 7 windows = 60840 tokens, no Muon), too large for the CPU oracle: the training-time program
+    must equal the step-by-step inference rollout (apply on the first window; then update on each clean window and
+    apply on it and the noisy window that follows, weights handed from call to call) -- both paths are checked
+    against the oracle at small sizes above.  bf16 bound 1e-2; gradients finite and linear in the upstream."""
+    b, d, dh, mb, ue = 2, 768, 1536, 4680, 9360
+    L = mb + 6 * ue
+    say("video model shape, full size", b, d, dh, L)
+    inp = O.make_inputs(b, L, d, dh, seed=5, act_dtype=torch.bfloat16, distinct_heads=2)
+    g = clone_to(inp, DEV)
+    go = torch.randn(b, L, d, generator=torch.Generator().manual_seed(3)).bfloat16().to(DEV)
+    names = [n for n in NAMES if g.get(n) is not None and n != "momentum"]
+
+    def run(upstream):
+        res = ar_video.ar_fast_weight_swish_glu_weight_norm_mini_batch(*args9(g), 1.0, 1, mb, -1, ue, False, 5, True)
+        return res, torch.autograd.grad(res[0], [g[n] for n in names], upstream)
+    res, g1 = run(go)
+    _, g2 = run(go * 2)
+    for n, a, c in zip(names, g1, g2):
+        assert torch.isfinite(a.float()).all(), n
+        assert O.rel_l2(c.float().cpu(), 2 * a.float().cpu()) < 5e-3, n
+    inf = ar_video.ar_fast_weight_swish_glu_weight_norm_mini_batch_inference
+    with torch.no_grad():
+        w = [g["w0"], g["w1"], g["w2"]]
+        sl = lambda t, a, e: t[:, a:e]
+        outs = [inf(*w, sl(g["q"], 0, mb), sl(g["k"], 0, mb), sl(g["v"], 0, mb), sl(g["lr0"], 0, mb), sl(g["lr1"], 0, mb),
+                    sl(g["lr2"], 0, mb), 1.0, 1, mb, False, False, 5, True)[0]]
+        for s0 in range(mb, L, ue):
+            r = inf(*w, sl(g["q"], s0, s0 + ue), sl(g["k"], s0, s0 + mb), sl(g["v"], s0, s0 + mb), sl(g["lr0"], s0, s0 + mb),
+                    sl(g["lr1"], s0, s0 + mb), sl(g["lr2"], s0, s0 + mb), 1.0, 1, mb, True, False, 5, True)
+            outs.append(r[0])
+            w = list(r[1:4])
+        e_out = O.rel_l2(torch.cat(outs, 1).cpu(), res[0].detach().cpu())
+        e_w = max(O.rel_l2(a.cpu(), c.detach().cpu()) for a, c in zip(w, res[1:4]))
+    say("   rollout vs program: out", e_out, "final weights", e_w)
+    assert e_out < 1e-2 and e_w < 2e-3
+
+
 # ---- size-independent properties at the benchmark size ----------------------------------------------
 def full_size_properties(b, L, d, dh, C, seed, single_update):
     inp = O.make_inputs(b, L, d, dh, seed=seed, act_dtype=torch.bfloat16, distinct_heads=4)
