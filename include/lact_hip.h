@@ -165,8 +165,12 @@ int lact_layer_post_backward(int32_t act_dtype, int32_t B, int32_t L, int32_t H,
  *   LACT_OPT_FUSED_NEWTON_SCHULZ: all Newton-Schulz iterations of an update (and of its backward) run as one
  *     kernel whose blocks meet at per-matrix barriers (bf16; rows and columns multiples of 192, of 128, or rows of
  *     128 and columns of 64; at most 8 iterations); otherwise three GEMM launches per iteration.
- * Returns the previous value (0 / 1), or -1 for an unknown option. */
-enum { LACT_OPT_STREAM_OVERLAP = 0, LACT_OPT_FUSED_NEWTON_SCHULZ = 1 };
+ *   LACT_OPT_NS_BARRIER_SPIN_LIMIT: how many polls a block of the fused Newton-Schulz kernel waits at a barrier
+ *     before it gives up (value <= 0 restores the default, a fraction of a second).  A block that gives up raises
+ *     an error word and goes on, so every kernel always ends; the step's results (weights, outputs that depend on
+ *     them, gradients) are then NaN.  Meant for tests of that path.
+ * Returns the previous value (0 / 1, or the previous limit), or -1 for an unknown option. */
+enum { LACT_OPT_STREAM_OVERLAP = 0, LACT_OPT_FUSED_NEWTON_SCHULZ = 1, LACT_OPT_NS_BARRIER_SPIN_LIMIT = 2 };
 int lact_set_option(int32_t option, int32_t value);
 
 /* Per-launch timing with HIP events on the caller's stream (no counterpart in the reference, which

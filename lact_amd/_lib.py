@@ -34,7 +34,7 @@ class Desc(Structure):
     ]
 
 
-OPT_STREAM_OVERLAP, OPT_FUSED_NEWTON_SCHULZ = 0, 1
+OPT_STREAM_OVERLAP, OPT_FUSED_NEWTON_SCHULZ, OPT_NS_BARRIER_SPIN_LIMIT = 0, 1, 2
 EXPORTS = ("lact_last_error", "lact_version", "lact_query_sizes", "lact_forward", "lact_forward_from_state", "lact_backward",
            "lact_newton_schulz_workspace_bytes", "lact_newton_schulz", "lact_set_option", "lact_profile_enable",
            "lact_profile_report", "lact_layer_pre_forward", "lact_layer_pre_backward", "lact_layer_lr_forward",

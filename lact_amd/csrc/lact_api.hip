@@ -135,6 +135,7 @@ struct SideCtx {
 };
 bool g_overlap = true;
 bool g_fused_ns = true;
+long long g_ns_spin_limit = NS_FUSED_SPIN_LIMIT;   // barrier wait bound of the fused Newton-Schulz kernels (lact_set_option)
 std::mutex g_enqueue_mutex;   // one program is enqueued at a time (the side-stream context is shared)
 SideCtx* side_ctx() {
   static SideCtx ctx[64];
@@ -511,6 +512,7 @@ struct Runner {
     p.r = B.r; p.c = B.c; p.S = P.S; p.nb = B.nb; p.mask = B.mask;
     for (int i = 0; i < 3 * P.S; ++i) p.coeffs[i] = P.coeffs[i];
     p.error = ns_error_word();
+    p.spin_limit = g_ns_spin_limit;
     const double terms = BWD ? 6.0 : 3.0;
     static const std::string name = std::string("k_ns_fused<") + std::to_string(TS::BM) + "x" + std::to_string(TS::BN) + (BWD ? ",bwd>" : ",fwd>");
     for (int z0 = 0; z0 < B.n; z0 += per) {
@@ -1411,6 +1413,11 @@ int lact_version(void) { return 1; }
 
 int lact_set_option(int32_t option, int32_t value) {
   std::lock_guard<std::mutex> lock(g_enqueue_mutex);
+  if (option == LACT_OPT_NS_BARRIER_SPIN_LIMIT) {
+    const long long was = g_ns_spin_limit;
+    g_ns_spin_limit = value > 0 ? value : NS_FUSED_SPIN_LIMIT;
+    return (int)std::min<long long>(was, 0x7fffffff);
+  }
   bool* flag = option == LACT_OPT_STREAM_OVERLAP ? &g_overlap : (option == LACT_OPT_FUSED_NEWTON_SCHULZ ? &g_fused_ns : nullptr);
   if (!flag) return fail("lact_set_option: unknown option");
   const int was = *flag ? 1 : 0;

@@ -32,7 +32,7 @@
 namespace lact {
 
 constexpr int NS_FUSED_MAX_STEPS = 8;
-constexpr long long NS_FUSED_SPIN_LIMIT = 4000000;   // polls of ~64 clocks: a fraction of a second
+constexpr long long NS_FUSED_SPIN_LIMIT = 4000000;   // default bound of a barrier wait, in polls of ~64 clocks: a fraction of a second
 
 struct NsFusedParams {
   int n, z0;                 // matrices of this launch: global indices z0 .. z0+n-1 of the packed [3b] arrays
@@ -58,14 +58,16 @@ struct NsFusedParams {
   float* dot_part; uint16_t* gc;
   unsigned* sync;            // [n][32] words, zeroed before the launch: word 0 = arrivals, word 1 = XCC id mask
   unsigned* error;           // set to 1 by a block whose barrier timed out
+  long long spin_limit;      // polls a block waits at a barrier before it gives up
 };
 
 struct GroupBarrier {
   unsigned* ctr;
   unsigned members, epoch;
+  long long limit;
   bool split;                // group spread over several XCDs: fence at device scope
-  __device__ __forceinline__ void init(unsigned* line, unsigned nmembers, unsigned* error) {
-    ctr = line; members = nmembers; epoch = 0; split = false;
+  __device__ __forceinline__ void init(unsigned* line, unsigned nmembers, unsigned* error, long long spin_limit) {
+    ctr = line; members = nmembers; epoch = 0; split = false; limit = spin_limit;
     unsigned xcc = 0;
     asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
     if (threadIdx.x == 0) __hip_atomic_fetch_or(line + 1, 1u << (xcc & 0xf), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -84,7 +86,7 @@ struct GroupBarrier {
       long long spins = 0;
       while (__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
         __builtin_amdgcn_s_sleep(1);
-        if (++spins > NS_FUSED_SPIN_LIMIT) {
+        if (++spins > limit) {
           __hip_atomic_store(error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           break;
         }
@@ -122,7 +124,7 @@ __global__ __launch_bounds__(DMA_THREADS) void k_ns_fused(const NsFusedParams p)
   if (group >= p.n) return;
   const int z = p.z0 + group;
   GroupBarrier bar;
-  bar.init(p.sync + (size_t)group * 32, nbm, p.error);
+  bar.init(p.sync + (size_t)group * 32, nbm, p.error, p.spin_limit);
   const bool sq_tile = member < tr * ts;             // this block owns a tile of the r x r stages
   const int sx = member / ts, sy = member % ts;      // its tile there
   const int rx = member / tc, ry = member % tc;      // its tile of the r x c stages

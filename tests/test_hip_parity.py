@@ -557,6 +557,39 @@ def test_video_model_shape_full_size_equals_its_inference_rollout():
     assert e_out < 1e-2 and e_w < 2e-3
 
 
+def test_fused_newton_schulz_barrier_timeout_ends_every_kernel_and_poisons_the_step():
+    """The blocks of the fused Newton-Schulz kernel wait for each other with a bounded poll.  The host forces the
+    bound to one poll: blocks give up at (nearly) every barrier, read partner tiles too early, raise the error word
+    -- and still run to their end.  The step's results must be NaN (never silently wrong numbers), and the next
+    call with the default bound must be right again."""
+    from lact_amd import _lib
+    say("fused Newton-Schulz: forced barrier timeout")
+    inp = problem(4, 3 * 128, 256, 256, 41, torch.bfloat16, momentum=True, lr_shift=-1.0)   # 4 or 8 blocks per matrix
+    hip, _ = block_causal_pair(128, True)
+
+    def run():
+        g = clone_to(inp, DEV)
+        out = hip(g)
+        go = torch.randn(out.shape, generator=torch.Generator().manual_seed(3)).bfloat16().to(DEV)
+        grads = grads_of(out, g, go)
+        torch.cuda.synchronize()
+        return out.detach().float().cpu(), {n: v.detach().float().cpu() for n, v in grads.items()}
+    good_out, good = run()
+    assert torch.isfinite(good_out).all()
+    L = _lib.lib()
+    prev = L.lact_set_option(_lib.OPT_NS_BARRIER_SPIN_LIMIT, 1)
+    try:
+        assert prev > 1
+        bad_out, bad = run()
+    finally:
+        assert L.lact_set_option(_lib.OPT_NS_BARRIER_SPIN_LIMIT, 0) == 1
+    assert torch.equal(bad_out[:, :128], good_out[:, :128])      # first chunk: initial weights, no Newton-Schulz yet
+    assert torch.isnan(bad_out[:, 128:]).all()                   # everything behind the first update
+    assert torch.isnan(bad["w0"]).all() and torch.isnan(bad["k"][:, :128]).all()
+    again_out, again = run()
+    assert torch.equal(again_out, good_out) and all(torch.equal(again[n], good[n]) for n in good)
+
+
 # ---- size-independent properties at the benchmark size ----------------------------------------------
 def full_size_properties(b, L, d, dh, C, seed, single_update):
     inp = O.make_inputs(b, L, d, dh, seed=seed, act_dtype=torch.bfloat16, distinct_heads=4)
