@@ -988,14 +988,28 @@ struct Runner {
     // gwcur: gradient w.r.t. the current weight version; "not valid" stands for zero (nothing written yet)
     bool gw_valid = dwf && (dwf[0] || dwf[1] || dwf[2]);
     if (gw_valid) LACT_LAUNCH("k_pack3", "k_pack3", 0.0, k_pack3, eg, dim3(256), s, gwcur, P.g.elems, d.b, dwf[0], dwf[1], dwf[2]);
-    // every gradient output is written in full by this call: rows that no step touches are zeroed here
-    // The small per-token arrays are added to by the steps, so they are cleared up front on the caller's stream.
-    // Rows of dq, dk, dv that no step writes are disjoint from everything the steps write: nothing waits for
-    // them, and they are cleared on the side stream -- unless ranges overlap partially, where the whole buffers
-    // start at zero and every step adds.
-    Touched seen_q, seen_kv;
+    // every gradient output is written in full by this call: rows that no step touches are zeroed here.
+    // Rows of dq, dk, dv and of the per-token arrays that no step writes are disjoint from everything the steps
+    // write: nothing waits for them, and they are cleared on the side stream -- unless ranges overlap partially,
+    // where the whole buffers start at zero and every step adds.  The momentum gradient is written by every
+    // update but the first of the program (which has no earlier state to weigh).
+    Touched seen_q, seen_kv, seen_m;
     const auto gaps_q = untouched(P.steps, LACT_APPLY, d.q_len, &seen_q.force);
     const auto gaps_kv = untouched(P.steps, LACT_UPDATE, d.kv_len, &seen_kv.force);
+    std::vector<lact_step_t> later_updates;
+    {
+      bool first = true;
+      for (auto& st : P.steps)
+        if (st.kind == LACT_UPDATE) {
+          if (!first) later_updates.push_back(st);
+          first = false;
+        }
+    }
+    auto gaps_m = untouched(later_updates, LACT_UPDATE, d.kv_len, &seen_m.force);
+    if (seen_kv.force) {
+      seen_m.force = true;
+      gaps_m.assign(1, std::make_pair(0, d.kv_len));
+    }
     const bool rows_on_side = !seen_q.force && !seen_kv.force && s_side != s_main;
     auto zero_rows = [&](hipStream_t zs) {
       ZeroList zl(d.b, zs);
@@ -1004,16 +1018,13 @@ struct Runner {
       for (auto& gp : gaps_kv) {
         zl.add(dk, (long long)d.kv_len * rowb, gp.first * rowb, (gp.second - gp.first) * rowb);
         zl.add(dv, (long long)d.kv_len * rowb, gp.first * rowb, (gp.second - gp.first) * rowb);
+        for (float* ptr : {dlr0, dlr1, dlr2})
+          zl.add(ptr, (long long)d.kv_len * 4, gp.first * 4LL, (gp.second - gp.first) * 4LL);
       }
+      for (auto& gp : gaps_m) zl.add(dmom, (long long)d.kv_len * 4, gp.first * 4LL, (gp.second - gp.first) * 4LL);
       zl.flush();
       return zl.launched;
     };
-    {
-      ZeroList zl(d.b, s);
-      float* small[4] = {dlr0, dlr1, dlr2, dmom};
-      for (float* ptr : small) zl.add(ptr, (long long)d.kv_len * 4, 0, (long long)d.kv_len * 4);
-      zl.flush();
-    }
     if (!rows_on_side) zero_rows(s_main);
     // The apply steps run on the side stream.  Their weight gradients go to gw_side[version & 1] and are added
     // by the consumer of that version's gradient (the renorm backward of the update that made the version, or
@@ -1239,7 +1250,7 @@ struct Runner {
           gm_valid = true;
           if (u > 0)
             LACT_LAUNCH("k_momentum_grad", "k_momentum_grad", 0.0, k_momentum_grad, dim3(d.b), dim3(256), s, scr<float>(P.t_mdot), P.nblk, d.b, dmom,
-                               (long long)d.kv_len, st.start, T_);
+                               (long long)d.kv_len, st.start, T_, seen_m.accumulate(st.start, st.end) ? 1 : 0);
         }
       } else if (P.momentum) {
         gm_valid = true;   // nothing was carried (first update of the program): as after the kernel above
@@ -1296,7 +1307,7 @@ struct Runner {
       LACT_LAUNCH("k_lr_reduce", "k_lr_reduce", 0.0, k_lr_reduce, dim3(ceil_div(T_, 256), d.b, 3), dim3(256), s, scr<float>(P.t_lrpart),
                          (long long)P.lr_slots * d.b * P.Tcap, (long long)d.b * P.Tcap,
                   lr_parts(), P.Tcap, dlr0, dlr1, dlr2,
-                         (long long)d.kv_len, st.start, T_);
+                         (long long)d.kv_len, st.start, T_, acc_kv ? 1 : 0);
       if (use_tail) {
         s = s_main;
         tail_ev = side->event();

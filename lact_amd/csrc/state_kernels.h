@@ -494,13 +494,16 @@ __global__ void k_grad_prep(const GradPrepParams p) {
 }
 
 // d loss / d momentum[t] = <g, M_prev> / chunk_len for every token of the chunk (mean, :172)
-__global__ void k_momentum_grad(const float* mdot_part, int nparts, int nb, float* dmom, long long bs, int start, int len) {
+__global__ void k_momentum_grad(const float* mdot_part, int nparts, int nb, float* dmom, long long bs, int start, int len, int accumulate) {
   const int ib = blockIdx.x;
   float s = 0.f;
   for (int j = 0; j < 3; ++j)
     for (int i = 0; i < nparts; ++i) s += mdot_part[(size_t)(j * nb + ib) * nparts + i];
   s /= (float)len;
-  for (int t = threadIdx.x; t < len; t += blockDim.x) dmom[ib * bs + start + t] += s;
+  for (int t = threadIdx.x; t < len; t += blockDim.x) {
+    float* dst = dmom + ib * bs + start + t;
+    *dst = accumulate ? *dst + s : s;
+  }
 }
 
 // out = coeff*in_add + sum of split partials; 4 elements per thread (total is a multiple of 4)
@@ -519,15 +522,16 @@ __global__ void k_reduce_partials(float* out, const float* in_add, float coeff, 
   st4(out + e, v);
 }
 
-// dlr_j[ib, start + t] += sum over slots of the row partials
+// dlr_j[ib, start + t] = (or +=, on rows an earlier step of this call wrote) sum over slots of the row partials
 __global__ void k_lr_reduce(const float* lrpart, long long mat_stride, long long slot_stride, int nslots, int Tcap,
-                            float* dlr0, float* dlr1, float* dlr2, long long bs, int start, int len) {
+                            float* dlr0, float* dlr1, float* dlr2, long long bs, int start, int len, int accumulate) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x, ib = blockIdx.y, j = blockIdx.z;
   if (t >= len) return;
   float s = 0.f;
   for (int i = 0; i < nslots; ++i) s += lrpart[j * mat_stride + i * slot_stride + (size_t)ib * Tcap + t];
   float* dst = j == 0 ? dlr0 : (j == 1 ? dlr1 : dlr2);
-  dst[ib * bs + start + t] += s;
+  dst += ib * bs + start + t;
+  *dst = accumulate ? *dst + s : s;
 }
 
 // final weight gradients: state gradient (+ accumulator carry) + the path through the initial row norms
