@@ -72,7 +72,7 @@ constexpr int DMA_BK = 64;
 // receives element (i & 3) of the 8 bytes addressed by lanes 4j + (i >> 2), j = 0..3 -- i.e. a 4(k) x 16(r)
 // patch comes back transposed, 4 consecutive k of one r per lane.  The rotation makes the four k-rows of a
 // patch land in different bank groups.
-constexpr int DMA_LOADERS = 2;     // loader waves per block
+constexpr int DMA_LOADERS = 4;     // loader waves per block
 template <int ROWS>
 struct DmaLane {
   static constexpr int NALL = ROWS / 8;            // copies per K-step, all loader waves together
@@ -230,9 +230,10 @@ struct DmaPipe {
   __device__ static __forceinline__ bool is_loader() { return __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) >= 4; }
 
   // ---- loader waves: every copy of every phase, split evenly.  MINLOADS: smallest per-K-step copy count of
-  // any phase (all loader waves together).  The count of outstanding vector-memory operations of a wave
-  // tops out at 63 -- one wave alone keeps at most 63 KiB in flight, which at 1-2 us of loaded memory
-  // latency caps a compute unit near 40 GB/s; two waves lift that cap above what the ring can hold.
+  // any phase (all loader waves together).  The copy rate of a compute unit grows with the number of waves that
+  // issue the copies, not only with the bytes in flight (measured with loads that hit the L2: 22 / 45 / 75 GB/s
+  // per compute unit from 2 / 4 / 8 issuing waves at the same depth), so four loader waves beside the four MFMA
+  // waves: eight waves are what the register budget of the MFMA waves (256 each) allows.
   template <int MINLOADS>
   __device__ __forceinline__ void load_all() {
     constexpr int PER_WAVE = MINLOADS / DMA_LOADERS;
