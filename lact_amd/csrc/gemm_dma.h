@@ -354,7 +354,7 @@ struct StageTile {
   static constexpr int LD = TS::BN + (E == 2 ? 8 : 4); // elements
   static constexpr int BYTES = TS::BM * LD * E;
   static constexpr int LPR = TS::BN / CH;              // lanes per row
-  static constexpr int RPP = TS::THREADS / LPR;        // rows per pass
+  static constexpr int RPP = DMA_THREADS / LPR;        // rows per pass: MFMA and loader waves all copy out
   static constexpr int PASSES = (TS::BM + RPP - 1) / RPP;
 
   // byte offset inside the tile of this lane's first quad (fragment 0,0, g = 0)
@@ -374,7 +374,7 @@ struct StageTile {
     Elem<uint16_t>::load4(reinterpret_cast<const uint16_t*>(base + frag_off(tm, tn, g)), o);
   }
   // this thread's position in the copy-out phase
-  __device__ static __forceinline__ bool active() { return (int)threadIdx.x < RPP * LPR; }   // RPP*LPR <= 256: loader wave idle
+  __device__ static __forceinline__ bool active() { return (int)threadIdx.x < RPP * LPR; }
   __device__ static __forceinline__ int row0() { return threadIdx.x / LPR; }
   __device__ static __forceinline__ int col0() { return (threadIdx.x % LPR) * CH; }
   // 16 bytes of copy-out pass `ps` for the thread whose first row is r0 (src = its address in pass 0); a pass
