@@ -38,18 +38,18 @@ CONFIGS = {
 # HBM bytes per launch at config 1 (read + write), from the FETCH_SIZE / WRITE_SIZE counters of two
 # `rocprofv3 --pmc` runs scaled by a 1 GiB copy (profiles/c1_fwd_bwd_hbm_traffic_pmc.txt); MiB.
 MEASURED_TRAFFIC_MIB = {
-    "k_ns_fused<192x192,bwd>": 768.9 + 361.4,
-    "k_ns_fused<192x192,fwd>": 438.1 + 386.9,
-    "k_token_reduce_dma<192x192>": 127.1 + 30.4,
-    "k_update_bwd_hidden_kept_dma": 151.5 + 74.2,
-    "k_apply_bwd_hidden_dma": 78.0 + 72.0,
-    "k_update_hidden_dma": 79.0 + 144.0,
+    "k_ns_fused<192x192,bwd>": 750.8 + 357.9,
+    "k_ns_fused<192x192,fwd>": 434.9 + 387.1,
+    "k_token_reduce_dma<192x192>": 127.0 + 30.4,
+    "k_update_bwd_hidden_kept_dma": 151.7 + 74.2,
+    "k_apply_bwd_hidden_dma": 77.9 + 72.0,
+    "k_update_hidden_dma": 79.1 + 144.0,
     "k_apply_hidden_dma": 33.2 + 24.0,
 }
 
 
 # Whole step at config 1, same two counter runs (last line of that profile): read + written MiB
-MEASURED_STEP_TRAFFIC_MIB = 2801.0 + 1649.0
+MEASURED_STEP_TRAFFIC_MIB = 2778.0 + 1646.0
 PEAK_HBM_GBPS = 8000.0
 
 
