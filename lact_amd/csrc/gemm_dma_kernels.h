@@ -650,14 +650,14 @@ __global__ __launch_bounds__(DMA_THREADS) void k_update_bwd_hidden_kept_dma(cons
 struct TokenReduceDmaParams : TokenReduceParams {
   TileMap map;   // token splits, output tiles, 3 * batch
 };
+// One block of the reduction; `lin` is the block's linear index in the reduction's tile map.
 template <class TS>
-__global__ __launch_bounds__(DMA_THREADS) void k_token_reduce_dma(const TokenReduceDmaParams p) {
-  extern __shared__ __attribute__((aligned(16))) char smem[];
+__device__ __forceinline__ void token_reduce_dma_block(const TokenReduceDmaParams& p, int lin, char* smem) {
   constexpr int STAGES = row_stages<TS>();
   using Pipe = DmaPipe<TS, 1, 2, STAGES>;
   int split, tile, bz;   // map: (splits, tiles, 3*nb)
-  clear_words(p.prep_clear, blockIdx.x == 0);
-  if (!p.map.locate(blockIdx.x, split, tile, bz)) return;
+  clear_words(p.prep_clear, lin == 0);
+  if (!p.map.locate(lin, split, tile, bz)) return;
   const int j = bz / p.nb, ib = bz % p.nb;
   const TokenReduceJob& job = p.job[j];
   const int tiles_n = (job.N + TS::BN - 1) / TS::BN;
@@ -771,6 +771,44 @@ __global__ __launch_bounds__(DMA_THREADS) void k_token_reduce_dma(const TokenRed
       dst += rstep;
     }
   }
+}
+
+template <class TS>
+__global__ __launch_bounds__(DMA_THREADS) void k_token_reduce_dma(const TokenReduceDmaParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  token_reduce_dma_block<TS>(p, blockIdx.x, smem);
+}
+
+// The token reduction of an update's backward together with the two token-row GEMMs that read the same
+// intermediates (dk: four terms, K-strided weights; dv: two terms): three independent pieces of work that, as
+// launches of their own, each end in a round of blocks that leaves most compute units idle.  One grid, longest
+// blocks first; every piece keeps its own tile map (the offsets are multiples of 8, so a block's XCD stays the
+// one its map assumes).
+struct TokenReduceRowsParams {
+  TokenReduceDmaParams tr;
+  RowGemmDmaParams<4> r4;
+  RowGemmDmaParams<2> r2;
+  int ntr, n4;   // blocks of the reduction and of the four-term GEMM
+};
+static_assert(sizeof(TokenReduceRowsParams) <= 4096, "kernel arguments must fit the 4 KiB argument segment");
+template <class TS>
+__global__ __launch_bounds__(DMA_THREADS) void k_token_reduce_rows_dma(const TokenReduceRowsParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  int lin = blockIdx.x;
+  if (lin < p.ntr) {
+    token_reduce_dma_block<TS>(p.tr, lin, smem);
+    return;
+  }
+  lin -= p.ntr;
+  int bx, by, z;
+  if (lin < p.n4) {
+    if (!p.r4.map.locate(lin, bx, by, z)) return;
+    row_gemm_tile<TS_ROW, 4, EPI_STORE, true, false>(p.r4, bx, by, z, smem);
+    return;
+  }
+  lin -= p.n4;
+  if (!p.r2.map.locate(lin, bx, by, z)) return;
+  row_gemm_tile<TS_ROW, 2, EPI_STORE, false, false>(p.r2, bx, by, z, smem);
 }
 
 }  // namespace lact

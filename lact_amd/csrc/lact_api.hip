@@ -642,8 +642,16 @@ struct Runner {
     float* m_ext[3];
     ClearWords clear;
   };
+  // `rows`: two token-row GEMMs (four and two terms, dk and dv of an update's backward) that may ride in the same
+  // launch as the asynchronous-copy reduction; `done` tells the caller whether they did.
+  struct RowCompanions {
+    RowGemmParams<4> r4;
+    RowGemmParams<2> r2;
+    bool done = false;
+  };
   int token_reduce(const char* site, const TokenReduceJob (&jobs)[3], int tokens, float* add_out = nullptr,
-                   const float* add_in = nullptr, float coeff = 0.f, const PrepFold* prep = nullptr) const {
+                   const float* add_in = nullptr, float coeff = 0.f, const PrepFold* prep = nullptr,
+                   RowCompanions* rows = nullptr) const {
     TokenReduceParams p;
     memset(&p, 0, sizeof(p));
     for (int i = 0; i < 3; ++i) p.job[i] = jobs[i];
@@ -672,7 +680,35 @@ struct Runner {
           for (int j = 0; j < 3; ++j) pd.prep_m_ext[j] = prep->m_ext[j];
         } else if (direct) { pd.add_out = add_out; pd.add_in = coeff != 0.f ? add_in : nullptr; pd.coeff = coeff; }
         else slots = sp.n;
-        if (big) {
+        bool with_rows = rows != nullptr && rows->r4.N % 8 == 0 && rows->r2.N % 8 == 0;
+        if (with_rows) {
+          for (int t = 0; t < 4; ++t) with_rows = with_rows && rows->r4.t[t].K % 64 == 0;
+          for (int t = 0; t < 2; ++t) with_rows = with_rows && rows->r2.t[t].K % 64 == 0;
+        }
+        if (with_rows) {
+          TokenReduceRowsParams q;
+          q.tr = pd;
+          q.r4.g = rows->r4; q.r4.out_ct = nullptr;
+          q.r4.map = make_tile_map(ceil_div(rows->r4.M, TS_ROW::BM), ceil_div(rows->r4.N, TS_ROW::BN), d.b);
+          q.r2.g = rows->r2; q.r2.out_ct = nullptr;
+          q.r2.map = make_tile_map(ceil_div(rows->r2.M, TS_ROW::BM), ceil_div(rows->r2.N, TS_ROW::BN), d.b);
+          q.ntr = pd.map.grid(); q.n4 = q.r4.map.grid();
+          const dim3 gr(q.ntr + q.n4 + q.r2.map.grid());
+          double frows = 0;
+          for (int t = 0; t < 4; ++t) frows += 2.0 * rows->r4.M * rows->r4.N * rows->r4.t[t].K * d.b;
+          for (int t = 0; t < 2; ++t) frows += 2.0 * rows->r2.M * rows->r2.N * rows->r2.t[t].K * d.b;
+          constexpr int SMR = cmax(DmaSmem<TS_ROW, 1, row_stages<TS_ROW>()>::BYTES, StageTile<TS_ROW, 4>::BYTES);
+          if (big) {
+            constexpr int SM = cmax(SMR, cmax(DmaSmem<TS_NS, 1, row_stages<TS_NS>()>::BYTES, StageTile<TS_NS, 4>::BYTES));
+            LACT_BIG_LDS(k_token_reduce_rows_dma<TS_NS>, SM);
+            LACT_LAUNCH_SMEM("k_token_reduce_rows_dma<192x192>", site, fl + frows, (k_token_reduce_rows_dma<TS_NS>), gr, dim3(DMA_THREADS), SM, s, q);
+          } else {
+            constexpr int SM = cmax(SMR, cmax(DmaSmem<TS_SQ, 1, row_stages<TS_SQ>()>::BYTES, StageTile<TS_SQ, 4>::BYTES));
+            LACT_BIG_LDS(k_token_reduce_rows_dma<TS_SQ>, SM);
+            LACT_LAUNCH_SMEM("k_token_reduce_rows_dma<128x128>", site, fl + frows, (k_token_reduce_rows_dma<TS_SQ>), gr, dim3(DMA_THREADS), SM, s, q);
+          }
+          rows->done = true;
+        } else if (big) {
           constexpr int SM = cmax(DmaSmem<TS_NS, 1, row_stages<TS_NS>()>::BYTES, StageTile<TS_NS, 4>::BYTES);
           LACT_BIG_LDS(k_token_reduce_dma<TS_NS>, SM);
           LACT_LAUNCH_SMEM("k_token_reduce_dma<192x192>", site, fl, (k_token_reduce_dma<TS_NS>), g, dim3(DMA_THREADS), SM, s, pd);
@@ -1286,6 +1322,10 @@ struct Runner {
         wait_for(s_tail, s_main);
         s = s_tail;
       }
+      // without that hand-over the two GEMMs share the launch of the token reduction below (when it runs on the
+      // asynchronous-copy kernel; otherwise they are launched after it)
+      RowCompanions rows_job;
+      const bool rows_ride = !use_tail && kBf16;
       {  // dk = (dgate*lr0) G0 + (dh2*lr2) G2 + gG W0 + gH2 W2
         auto p = row_params<4>();
         set_term(p.t[0], z0, d.dh, zbs, g0, d.d, P.g.elems, d.dh);
@@ -1294,7 +1334,8 @@ struct Runner {
         set_term(p.t[3], h(2), d.dh, hbs(), wc(vprev, 2), d.d, P.g.elems, d.dh);
         p.M = T_; p.N = d.d; p.out = dk + (size_t)st.start * d.d; p.ldo = d.d; p.bso = (long long)d.kv_len * d.d;
         p.accumulate = acc_kv;
-        launch_row_gemm<T, false, 4, EPI_STORE>("update_bwd_dk", p, d.b, s, true);
+        if (use_tail || !kBf16) launch_row_gemm<T, false, 4, EPI_STORE>("update_bwd_dk", p, d.b, s, true);
+        rows_job.r4 = p;
       }
       {  // dv = (hidden*lr1) G1^T + gDH W1^T
         auto p = row_params<2>();
@@ -1302,7 +1343,8 @@ struct Runner {
         set_term(p.t[1], h(1), d.dh, hbs(), wc(vprev, 1), d.dh, P.g.elems, d.dh);
         p.M = T_; p.N = d.d; p.out = dv + (size_t)st.start * d.d; p.ldo = d.d; p.bso = (long long)d.kv_len * d.d;
         p.accumulate = acc_kv;
-        launch_row_gemm<T, true, 2, EPI_STORE>("update_bwd_dv", p, d.b, s, true);
+        if (use_tail || !kBf16) launch_row_gemm<T, true, 2, EPI_STORE>("update_bwd_dv", p, d.b, s, true);
+        rows_job.r2 = p;
       }
       LACT_LAUNCH("k_lr_reduce", "k_lr_reduce", 0.0, k_lr_reduce, dim3(ceil_div(T_, 256), d.b, 3), dim3(256), s, scr<float>(P.t_lrpart),
                          (long long)P.lr_slots * d.b * P.Tcap, (long long)d.b * P.Tcap,
@@ -1325,9 +1367,14 @@ struct Runner {
         jobs[2].M = d.dh; jobs[2].N = d.d;
         set_tr_term(jobs[2].t[0], h(2), d.dh, hbs(), kc, d.k_ld, d.k_bs);
         const float pass = d.prenorm ? 0.f : ((P.muon && d.muon_replaces_weight) ? 0.f : 1.f);
-        if (const int ns_ = token_reduce("update_bwd_dw", jobs, T_, gwcur, gwhat, pass))
+        if (const int ns_ = token_reduce(rows_ride ? "update_bwd_dw_dk_dv" : "update_bwd_dw", jobs, T_, gwcur, gwhat, pass, nullptr,
+                                         rows_ride ? &rows_job : nullptr))
           LACT_LAUNCH("k_reduce_partials", "k_reduce_partials", 0.0, k_reduce_partials, flat, dim3(256), s, gwcur, pass != 0.f ? gwhat : nullptr, pass, partial, ns_, (long long)P.mat3);
         gw_valid = true;
+        if (rows_ride && !rows_job.done) {
+          launch_row_gemm<T, false, 4, EPI_STORE>("update_bwd_dk", rows_job.r4, d.b, s, true);
+          launch_row_gemm<T, true, 2, EPI_STORE>("update_bwd_dv", rows_job.r2, d.b, s, true);
+        }
       }
       --ver;
     }
