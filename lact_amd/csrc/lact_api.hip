@@ -775,6 +775,23 @@ struct Runner {
       p.wc = P.bf16 ? (void*)wc(0) : nullptr;
       LACT_LAUNCH("k_init_state", "k_init_state", 0.0, (k_init_state<T>), rowgrid, dim3(256), s, p);
     }
+    // mean of the momentum over the chunk of every update that weighs an earlier state (the first update of a
+    // program has none unless the caller carried one in): they depend on the input only -- one launch up front
+    if (P.momentum) {
+      int u0 = P.state_in ? 0 : 1, ui = 0, n = 0;
+      MomentumMeanRanges r;
+      auto flush = [&]() {
+        if (n > 0) LACT_LAUNCH("k_momentum_mean", "k_momentum_mean", 0.0, k_momentum_mean, dim3(d.b, n), dim3(256), s, mom, (long long)d.kv_len, r, mbar(u0));
+        u0 += n; n = 0;
+      };
+      for (const auto& st : P.steps) {
+        if (st.kind != LACT_UPDATE) continue;
+        if (ui++ < u0) continue;
+        r.start[n] = st.start; r.len[n] = st.end - st.start;
+        if (++n == 256) flush();
+      }
+      flush();
+    }
     int ver = 0, u = 0;
     T* upd_z[3] = {nullptr, nullptr, nullptr};   // lr-scaled operands of the current update's gradient GEMMs
     long long upd_zbs = 0;
@@ -830,8 +847,6 @@ struct Runner {
         launch_hidden(1, hp, ver, T_);
         upd_z[0] = z0; upd_z[1] = z1; upd_z[2] = z2; upd_zbs = zbs;
       }
-      // mean of the momentum over the chunk (weighs the earlier state; the first update has none: never used)
-      if (has_prev(u)) LACT_LAUNCH("k_momentum_mean", "k_momentum_mean", 0.0, k_momentum_mean, dim3(d.b), dim3(256), s, mom, (long long)d.kv_len, st.start, T_, mbar(u));
       int dw_slots = 0;
       {
         TokenReduceJob jobs[3];

@@ -96,13 +96,18 @@ __global__ void k_init_state(const InitParams p) {
 }
 
 // ---- mean of the per-token momentum over one chunk (ttt_operation.py:171-172) --------------------
-__global__ void k_momentum_mean(const float* mom, long long bs, int start, int len, float* mbar) {
+// One launch for the chunks of up to 256 updates: grid (batch, chunks), mbar [chunks][batch].
+struct MomentumMeanRanges {
+  int start[256], len[256];
+};
+__global__ void k_momentum_mean(const float* mom, long long bs, const MomentumMeanRanges r, float* mbar) {
   __shared__ float red[16];
+  const int start = r.start[blockIdx.y], len = r.len[blockIdx.y];
   const float* m = mom + blockIdx.x * bs + start;
   float s = 0.f;
   for (int t = threadIdx.x; t < len; t += blockDim.x) s += m[t];
   s = block_sum(s, red);
-  if (threadIdx.x == 0) mbar[blockIdx.x] = s / (float)len;
+  if (threadIdx.x == 0) mbar[(size_t)blockIdx.y * gridDim.x + blockIdx.x] = s / (float)len;
 }
 
 // ---- reduce split partials, add momentum, emit the bf16 Newton-Schulz input ---------------------
