@@ -312,7 +312,7 @@ struct Plan {
     t_xbtmp = sc.take(mat3 * nsz);
     t_ss = sc.take((size_t)3 * d.b * nblk * 4);
     t_dot = sc.take((size_t)3 * d.b * std::max(nblk, 32) * 4);   // partial dots: per chunk of a matrix, or per block of the fused kernel
-    t_mdot = sc.take((size_t)3 * d.b * nblk * 4);
+    t_mdot = sc.take((size_t)std::max(1, nupd) * 3 * d.b * nblk * 4);   // one slot per update: the momentum gradients are written at the end
     for (int i = 0; i < 2; ++i) t_gwhat[i] = sc.take(mat3 * 4);
     t_gwcur = sc.take(mat3 * 4);
     t_gmcarry = sc.take(mat3 * 4);
@@ -1061,6 +1061,13 @@ struct Runner {
       seen_m.force = true;
       gaps_m.assign(1, std::make_pair(0, d.kv_len));
     }
+    // momentum gradients: one launch at the end for all updates, unless token ranges of (later) updates repeat
+    bool mg_each = seen_m.force;
+    for (size_t i = 0; i < later_updates.size() && !mg_each; ++i)
+      for (size_t j = i + 1; j < later_updates.size(); ++j)
+        if (later_updates[i].start < later_updates[j].end && later_updates[j].start < later_updates[i].end) mg_each = true;
+    std::vector<int> mg_updates;
+    std::vector<std::pair<int, int>> mg_ranges;
     const bool rows_on_side = !seen_q.force && !seen_kv.force && s_side != s_main;
     auto zero_rows = [&](hipStream_t zs) {
       ZeroList zl(d.b, zs);
@@ -1294,14 +1301,25 @@ struct Runner {
         p.m_prev = (P.momentum && u > 0) ? dsave(u - 1) : nullptr;
         p.mbar = (P.momentum && u > 0) ? mbar(u) : nullptr;
         p.gc = scr<T>(P.t_gc);
-        p.mdot_part = scr<float>(P.t_mdot);
+        p.mdot_part = scr<float>(P.t_mdot) + (size_t)u * 3 * d.b * P.nblk;
         if (P.muon && ns_fused_any()) p.poison = ns_error_word();
         LACT_LAUNCH("k_grad_prep", "k_grad_prep", 0.0, (k_grad_prep<T, TN>), dim3(P.nblk, 3 * d.b), dim3(256), s, p);
         if (P.momentum) {
           gm_valid = true;
-          if (u > 0)
-            LACT_LAUNCH("k_momentum_grad", "k_momentum_grad", 0.0, k_momentum_grad, dim3(d.b), dim3(256), s, scr<float>(P.t_mdot), P.nblk, d.b, dmom,
-                               (long long)d.kv_len, st.start, T_, seen_m.accumulate(st.start, st.end) ? 1 : 0);
+          // the gradient of the per-token momentum needs these dot products only: written by one launch at the end
+          // (by one launch per update, in this order, when token ranges repeat and their shares add up)
+          if (u > 0) {
+            const bool acc = seen_m.accumulate(st.start, st.end);
+            if (acc || mg_each) {
+              MomentumMeanRanges r1;
+              r1.start[0] = st.start; r1.len[0] = T_;
+              LACT_LAUNCH("k_momentum_grad", "k_momentum_grad", 0.0, k_momentum_grad, dim3(d.b, 1), dim3(256), s, scr<float>(P.t_mdot) + (size_t)u * 3 * d.b * P.nblk,
+                          0LL, P.nblk, d.b, dmom, (long long)d.kv_len, r1, acc ? 1 : 0);
+            } else {
+              mg_updates.push_back(u);
+              mg_ranges.emplace_back(st.start, T_);
+            }
+          }
         }
       } else if (P.momentum) {
         gm_valid = true;   // nothing was carried (first update of the program): as after the kernel above
@@ -1392,6 +1410,22 @@ struct Runner {
         }
       }
       --ver;
+    }
+    if (!mg_updates.empty()) {
+      // deferred updates are all updates but the first, met in descending order: slot u - 1 of the launch is update u
+      const size_t slot = (size_t)3 * d.b * P.nblk;
+      const int total = (int)mg_updates.size();
+      for (int i0 = 0; i0 < total; i0 += 256) {
+        const int n = std::min(256, total - i0);
+        MomentumMeanRanges r;
+        int umin = mg_updates[total - 1 - i0];
+        for (int i = 0; i < n; ++i) {
+          const int idx = total - 1 - (i0 + i);   // ascending update index
+          r.start[i] = mg_ranges[idx].first; r.len[i] = mg_ranges[idx].second;
+        }
+        LACT_LAUNCH("k_momentum_grad", "k_momentum_grad", 0.0, k_momentum_grad, dim3(d.b, n), dim3(256), s, scr<float>(P.t_mdot) + (size_t)umin * slot,
+                    (long long)slot, P.nblk, d.b, dmom, (long long)d.kv_len, r, 0);
+      }
     }
     {
       FinishParams p;

@@ -498,12 +498,17 @@ __global__ void k_grad_prep(const GradPrepParams p) {
   }
 }
 
-// d loss / d momentum[t] = <g, M_prev> / chunk_len for every token of the chunk (mean, :172)
-__global__ void k_momentum_grad(const float* mdot_part, int nparts, int nb, float* dmom, long long bs, int start, int len, int accumulate) {
+// d loss / d momentum[t] = <g, M_prev> / chunk_len for every token of the chunk (mean, :172).  Grid (batch, updates):
+// update i of the launch has its partial dot products at mdot_part + i * slot_stride and the token range r[i]; the
+// ranges of one launch do not overlap (each row is written by one block).
+__global__ void k_momentum_grad(const float* mdot_part, long long slot_stride, int nparts, int nb, float* dmom, long long bs,
+                                const MomentumMeanRanges r, int accumulate) {
   const int ib = blockIdx.x;
+  const float* part = mdot_part + blockIdx.y * slot_stride;
+  const int start = r.start[blockIdx.y], len = r.len[blockIdx.y];
   float s = 0.f;
   for (int j = 0; j < 3; ++j)
-    for (int i = 0; i < nparts; ++i) s += mdot_part[(size_t)(j * nb + ib) * nparts + i];
+    for (int i = 0; i < nparts; ++i) s += part[(size_t)(j * nb + ib) * nparts + i];
   s /= (float)len;
   for (int t = threadIdx.x; t < len; t += blockDim.x) {
     float* dst = dmom + ib * bs + start + t;
