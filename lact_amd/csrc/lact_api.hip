@@ -194,6 +194,7 @@ struct Plan {
   std::vector<NsBatch> nsb;
   size_t sq_total = 0;    // elements of one [r, r]-shaped buffer over all batches
   std::vector<lact_step_t> steps;
+  std::vector<lact_step_t> live;    // the steps that are executed: `steps` without the apply rows a later step overwrites
   std::vector<float> coeffs;
   MatGeom g;
   int nupd = 0, Tcap = 0, S = -1, esz = 2, nsz = 2, r = 0, c = 0, nblk = 1, lr_slots = 1, tiles = 1, nsplit_max = 1;
@@ -251,6 +252,35 @@ struct Plan {
         if (s.out_start < 0 || s.out_start + (s.end - s.start) > d.out_len) return fail("apply output range exceeds out_len");
       }
       Tcap = std::max(Tcap, s.end - s.start);
+    }
+    // Output rows that a later apply step writes again are dead in the earlier one (the reference's slice
+    // assignment lets the later write win, and no gradient reaches the overwritten values): every apply step is
+    // cut down to the rows that survive, in the forward and in the backward alike.  What is left never writes a
+    // row twice, so the apply steps may run in any order.
+    live.clear();
+    for (size_t i = 0; i < steps.size(); ++i) {
+      const lact_step_t& a = steps[i];
+      if (a.kind != LACT_APPLY) { live.push_back(a); continue; }
+      std::vector<std::pair<int, int>> keep(1, std::make_pair(a.out_start, a.out_start + (a.end - a.start)));
+      for (size_t j = i + 1; j < steps.size() && !keep.empty(); ++j) {
+        const lact_step_t& b = steps[j];
+        if (b.kind != LACT_APPLY) continue;
+        const int b0 = b.out_start, b1 = b.out_start + (b.end - b.start);
+        std::vector<std::pair<int, int>> next;
+        for (auto& iv : keep) {
+          if (b1 <= iv.first || iv.second <= b0) { next.push_back(iv); continue; }
+          if (iv.first < b0) next.emplace_back(iv.first, b0);
+          if (b1 < iv.second) next.emplace_back(b1, iv.second);
+        }
+        keep.swap(next);
+      }
+      for (auto& iv : keep) {
+        lact_step_t c = a;
+        c.start = a.start + (iv.first - a.out_start);
+        c.end = c.start + (iv.second - iv.first);
+        c.out_start = iv.first;
+        live.push_back(c);
+      }
     }
     g.d = d.d;
     g.dh = d.dh;
@@ -784,7 +814,7 @@ struct Runner {
         if (n > 0) LACT_LAUNCH("k_momentum_mean", "k_momentum_mean", 0.0, k_momentum_mean, dim3(d.b, n), dim3(256), s, mom, (long long)d.kv_len, r, mbar(u0));
         u0 += n; n = 0;
       };
-      for (const auto& st : P.steps) {
+      for (const auto& st : P.live) {
         if (st.kind != LACT_UPDATE) continue;
         if (ui++ < u0) continue;
         r.start[n] = st.start; r.len[n] = st.end - st.start;
@@ -823,7 +853,7 @@ struct Runner {
       }
       pending.clear();
     };
-    for (const auto& st : P.steps) {
+    for (const auto& st : P.live) {
       const int T_ = st.end - st.start;
       if (st.kind == LACT_APPLY) {
         pending.emplace_back(&st, ver);
@@ -1045,12 +1075,12 @@ struct Runner {
     // where the whole buffers start at zero and every step adds.  The momentum gradient is written by every
     // update but the first of the program (which has no earlier state to weigh).
     Touched seen_q, seen_kv, seen_m;
-    const auto gaps_q = untouched(P.steps, LACT_APPLY, d.q_len, &seen_q.force);
-    const auto gaps_kv = untouched(P.steps, LACT_UPDATE, d.kv_len, &seen_kv.force);
+    const auto gaps_q = untouched(P.live, LACT_APPLY, d.q_len, &seen_q.force);
+    const auto gaps_kv = untouched(P.live, LACT_UPDATE, d.kv_len, &seen_kv.force);
     std::vector<lact_step_t> later_updates;
     {
       bool first = true;
-      for (auto& st : P.steps)
+      for (auto& st : P.live)
         if (st.kind == LACT_UPDATE) {
           if (!first) later_updates.push_back(st);
           first = false;
@@ -1112,8 +1142,8 @@ struct Runner {
     int ver = P.nupd, u = P.nupd;
     int carry_main = -1;       // index of the gwhat buffer holding the accumulator's gradient (pre-norm)
     bool gm_valid = false;     // gmcarry holds d loss / d (momentum state after update u-1)
-    for (int si = (int)P.steps.size() - 1; si >= 0; --si) {
-      const lact_step_t& st = P.steps[si];
+    for (int si = (int)P.live.size() - 1; si >= 0; --si) {
+      const lact_step_t& st = P.live[si];
       const int T_ = st.end - st.start;
       if (st.kind == LACT_APPLY) {
         const T* qc = q + (size_t)st.start * d.q_ld;

@@ -369,21 +369,23 @@ def test_nvs_config3_shape_forward():
 
 
 # ---- AR-video schedule -----------------------------------------------------------------------------
-@pytest.mark.parametrize("use_momentum,weight_norm,use_moun", [(False, True, True), (True, False, False), (True, True, True)])
-def test_ar_video_interleaved(use_momentum, weight_norm, use_moun):
-    say("ar video", use_momentum, weight_norm, use_moun)
+@pytest.mark.parametrize("use_momentum,weight_norm,use_moun,repeat", [
+    (False, True, True, 1), (True, False, False, 1), (True, True, True, 1),
+    (True, True, False, 2)])      # every chunk updated twice: k, v, lr and momentum gradients of a chunk add up
+def test_ar_video_interleaved(use_momentum, weight_norm, use_moun, repeat):
+    say("ar video", use_momentum, weight_norm, use_moun, repeat)
     b, d, dh, mb, L = 2, 64, 128, 40, 240
     inp = problem(b, L, d, dh, 14, torch.bfloat16, momentum=use_momentum)
 
     def hip(t):
         r = ar_video.ar_fast_weight_swish_glu_weight_norm_mini_batch_with_momentum(
-            *args9(t), 0.5, 1, mb, -1, 2 * mb, use_moun, 3, weight_norm, t["momentum"], use_momentum)
+            *args9(t), 0.5, repeat, mb, -1, 2 * mb, use_moun, 3, weight_norm, t["momentum"], use_momentum)
         assert len(r) == 4
         return r[0]
 
     def orc(t, num):
         return O.ar_fast_weight_swish_glu_weight_norm_mini_batch(
-            *args9(t), 0.5, 1, mb, -1, 2 * mb, use_moun, 3, weight_norm, t["momentum"], use_momentum, num=num)[0]
+            *args9(t), 0.5, repeat, mb, -1, 2 * mb, use_moun, 3, weight_norm, t["momentum"], use_momentum, num=num)[0]
     res, ref, r64 = run_both(hip, orc, inp, AC, ref64=True)
     if use_moun:
         assert_within_noise_floor(res, ref, r64, "ar-video")
@@ -591,6 +593,27 @@ def test_fused_newton_schulz_barrier_timeout_ends_every_kernel_and_poisons_the_s
     assert torch.isnan(bad["w0"]).all() and torch.isnan(bad["k"][:, :128]).all()
     again_out, again = run()
     assert torch.equal(again_out, good_out) and all(torch.equal(again[n], good[n]) for n in good)
+
+
+@pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
+def test_output_rows_written_twice_belong_to_the_later_apply(act):
+    """A program may write an output row in several apply steps; the reference's slice assignment lets the last
+    write win and autograd sends the overwritten values no gradient.  Here: rows 48..112 are written by the first
+    apply (initial weights) and again by the second (updated weights), rows 112..160 only by the second, and a
+    third apply rewrites 0..16 -- forward and every gradient against the oracle."""
+    say("overwritten output rows", act)
+    b, L, d, dh = 2, 160, 64, 128
+    inp = problem(b, L, d, dh, 52, act, momentum=True, lr_shift=-1.0)
+    prog_steps = ((LACT_APPLY, 0, 112, 0), (ops.LACT_UPDATE, 0, 64, 0), (LACT_APPLY, 48, 160, 48),
+                  (ops.LACT_UPDATE, 64, 128, 0), (LACT_APPLY, 0, 16, 0))
+    prog = ops.Program(steps=prog_steps, out_len=L)
+    hip = lambda t: ops.run_program(prog, *args9(t), t["momentum"])[0]
+    osteps = [O.Step(O.APPLY if k == LACT_APPLY else O.UPDATE, s0, e0) for k, s0, e0, _ in prog_steps]
+    orc = lambda t, num: O.run_program(*args9(t), osteps, num=num, momentum=t["momentum"])[0]
+    res, ref = run_both(hip, orc, inp, PLAIN if act == torch.float32 else AC)
+    errs = compare(res, ref)
+    say("  ", errs)
+    assert max(errs.values()) < (1e-4 if act == torch.float32 else 1e-2)
 
 
 # ---- size-independent properties at the benchmark size ----------------------------------------------
