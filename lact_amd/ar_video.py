@@ -27,7 +27,7 @@ def _ar_steps(seq_len, q_len, mini_batch_size, update_length, update_every, num_
     steps = [(LACT_APPLY, 0, first, 0)]
     for _ in range(num_repeat):
         for s in range(first, update_length, update_every):
-            steps.append((LACT_UPDATE, s, s + mini_batch_size, 0))
+            steps.append((LACT_UPDATE, s, min(s + mini_batch_size, seq_len), 0))   # slices stop at the end (:79-82)
             steps.append((LACT_APPLY, s, min(s + update_every, q_len), s))
     return tuple(steps)
 
@@ -59,7 +59,7 @@ def ar_fast_weight_swish_glu_weight_norm_mini_batch_inference(
         w0, w1, w2, q, k, v, lr0, lr1, lr2, w_scale: float, num_repeat: int = 1, mini_batch_size: int = -1,
         do_update: bool = False, use_moun: bool = False, num_moun_iters: int = 3, weight_norm: bool = True):
     """ar_lact_swa_repeat.py:172-296: optional repeated update on the first mini-batch, then apply on all q."""
-    mb = k.shape[1] if mini_batch_size == -1 else mini_batch_size
+    mb = k.shape[1] if mini_batch_size == -1 else min(mini_batch_size, k.shape[1])
     steps = [(LACT_UPDATE, 0, mb, 0)] * (num_repeat if do_update else 0) + [(LACT_APPLY, 0, q.shape[1], 0)]
     prog = Program(steps=tuple(steps), out_len=q.shape[1],
                    ns_coeffs=(NS_CLASSIC,) * num_moun_iters if use_moun else None,
@@ -76,7 +76,7 @@ def ar_fast_weight_swish_glu_weight_norm_mini_batch_inference_with_momentum(
         use_momentum: bool = False):
     """ar_lact_swa_repeat_sp.py:197-339.  Returns (output, w0, w1, w2, m0, m1, m2): the momentum states go in and
     come out, so that the caller can keep them between denoising steps.  Inference only (torch.no_grad)."""
-    mb = k.shape[1] if mini_batch_size == -1 else mini_batch_size
+    mb = k.shape[1] if mini_batch_size == -1 else min(mini_batch_size, k.shape[1])
     updates = num_repeat if do_update else 0
     steps = [(LACT_UPDATE, 0, mb, 0)] * updates + [(LACT_APPLY, 0, q.shape[1], 0)]
     prog = Program(steps=tuple(steps), out_len=q.shape[1],

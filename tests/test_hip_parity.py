@@ -372,20 +372,21 @@ def test_nvs_config3_shape_forward():
 @pytest.mark.parametrize("use_momentum,weight_norm,use_moun,repeat", [
     (False, True, True, 1), (True, False, False, 1), (True, True, True, 1),
     (True, True, False, 2)])      # every chunk updated twice: k, v, lr and momentum gradients of a chunk add up
-def test_ar_video_interleaved(use_momentum, weight_norm, use_moun, repeat):
-    say("ar video", use_momentum, weight_norm, use_moun, repeat)
-    b, d, dh, mb, L = 2, 64, 128, 40, 240
+@pytest.mark.parametrize("L,update_length", [(240, -1), (230, -1), (240, 130)])   # whole windows; a cut last window; updates stop early
+def test_ar_video_interleaved(use_momentum, weight_norm, use_moun, repeat, L, update_length):
+    say("ar video", use_momentum, weight_norm, use_moun, repeat, L, update_length)
+    b, d, dh, mb = 2, 64, 128, 40
     inp = problem(b, L, d, dh, 14, torch.bfloat16, momentum=use_momentum)
 
     def hip(t):
         r = ar_video.ar_fast_weight_swish_glu_weight_norm_mini_batch_with_momentum(
-            *args9(t), 0.5, repeat, mb, -1, 2 * mb, use_moun, 3, weight_norm, t["momentum"], use_momentum)
+            *args9(t), 0.5, repeat, mb, update_length, 2 * mb, use_moun, 3, weight_norm, t["momentum"], use_momentum)
         assert len(r) == 4
         return r[0]
 
     def orc(t, num):
         return O.ar_fast_weight_swish_glu_weight_norm_mini_batch(
-            *args9(t), 0.5, repeat, mb, -1, 2 * mb, use_moun, 3, weight_norm, t["momentum"], use_momentum, num=num)[0]
+            *args9(t), 0.5, repeat, mb, update_length, 2 * mb, use_moun, 3, weight_norm, t["momentum"], use_momentum, num=num)[0]
     res, ref, r64 = run_both(hip, orc, inp, AC, ref64=True)
     if use_moun:
         assert_within_noise_floor(res, ref, r64, "ar-video")
