@@ -50,6 +50,7 @@ struct DmaOperand {
   int ld;
   int rows;              // valid rows from base on (may exceed the tile); multiple of 8 when ks
   int ks;
+  int ktail = 0;         // K-strided only: valid k rows of the last K-step when K is not a multiple of 64 (0: all 64)
 };
 
 // One phase: acc[j] += A * B_j^T over K, j < nb.
@@ -108,6 +109,32 @@ struct DmaLane {
     const uint16_t* b = base + kt * kstride;
 #pragma unroll
     for (int ii = 0; ii < N; ++ii) dma16<SC1>(b, voff[ii], lds_tile + ii * DMA_LOADERS * 1024);
+  }
+  // The last K-step of a K-strided operand whose K ends inside it (op.ktail valid k rows): the k rows past the end
+  // are read from the last valid one instead -- never past the operand.  Offsets computed here, once per phase.
+  template <bool SC1>
+  __device__ __forceinline__ void issue_tail(int kt, uint32_t lds_tile, const DmaOperand& op, int lw) const {
+    const int lane = threadIdx.x & 63;
+    const uint16_t* b = base + kt * kstride;
+#pragma unroll
+    for (int ii = 0; ii < N; ++ii) {
+      const int L = (lw + ii * DMA_LOADERS) * 64 + lane, k = min(L / G, op.ktail - 1), p = L % G;
+      int g = (p + G - (4 * ((L / G) & 3)) % G) % G;
+      g = min(g, op.rows / 8 - 1);
+      dma16<SC1>(b, (uint32_t)(((size_t)k * op.ld + g * 8) * 2), lds_tile + ii * DMA_LOADERS * 1024);
+    }
+  }
+  // The k rows past the end of K in the K-strided tile that has landed at `tile` (LDS; ktail valid k rows): cleared,
+  // so that whatever the other operand holds there adds nothing.  Every wave clears inside the chunks it copied
+  // itself (it has waited for exactly those).
+  __device__ static __forceinline__ void clear_tail(char* tile, int lw, int ktail) {
+    const int lane = threadIdx.x & 63;
+    const int first = ktail * ROWS * 2;   // first byte of the tile that lies past the end of K
+#pragma unroll
+    for (int ii = 0; ii < N; ++ii) {
+      const int off = (lw + ii * DMA_LOADERS) * 1024 + lane * 16;
+      if (off >= first) *reinterpret_cast<uint4*>(tile + off) = make_uint4(0, 0, 0, 0);
+    }
   }
 };
 
@@ -214,7 +241,8 @@ constexpr int DMA_THREADS = 256 + 64 * DMA_LOADERS;   // four MFMA waves + the l
 // only read fragments and issue MFMAs.  One barrier per K-step:
 //     loader:    wait until stage kt has landed; barrier; refill the stage the MFMA waves just left
 //     consumers: barrier; MFMAs on stage kt
-template <class TS, int NBMAX, int NPH, int STAGES, bool SC1 = false>
+// TAILS: a K-strided A operand may end inside its last K-step (DmaOperand::ktail), together with its B operand.
+template <class TS, int NBMAX, int NPH, int STAGES, bool SC1 = false, bool TAILS = false>
 struct DmaPipe {
   using SM = DmaSmem<TS, NBMAX, STAGES>;
   static constexpr int loads(int nb) { return (TS::BM + nb * TS::BN) / 8; }   // loader copies per K-step
@@ -257,10 +285,26 @@ struct DmaPipe {
     };
     auto issue_stage = [&]() {
       const uint32_t base = lds_addr(smem + (issued % STAGES) * SM::STAGE) + lw * 1024;
-      la.template issue<SC1>(ckt, base);
+      bool tail = false;
+      if constexpr (TAILS) {
+        if (ckt + 1 == cnk) {
 #pragma unroll
-      for (int j = 0; j < NBMAX; ++j)
-        if (j < cnb) lb[j].template issue<SC1>(ckt, base + SM::A_BYTES + j * SM::B_BYTES);
+          for (int i = 0; i < NPH; ++i)
+            if (i == cp && ph[i].a.ks && ph[i].a.ktail > 0) {
+              tail = true;
+              la.template issue_tail<SC1>(ckt, base, ph[i].a, lw);
+#pragma unroll
+              for (int j = 0; j < NBMAX; ++j)
+                if (j < cnb) lb[j].template issue_tail<SC1>(ckt, base + SM::A_BYTES + j * SM::B_BYTES, ph[i].b[j], lw);
+            }
+        }
+      }
+      if (!tail) {
+        la.template issue<SC1>(ckt, base);
+#pragma unroll
+        for (int j = 0; j < NBMAX; ++j)
+          if (j < cnb) lb[j].template issue<SC1>(ckt, base + SM::A_BYTES + j * SM::B_BYTES);
+      }
       ++issued;
       if (++ckt == cnk)
         while (cp + 1 < NPH) {
@@ -270,9 +314,25 @@ struct DmaPipe {
     };
     do next_phase(); while (cnk == 0 && cp + 1 < NPH);
     for (int i = 0; i < STAGES - 1 && issued < total; ++i) issue_stage();
+    // TAILS: the stage that holds a phase's ragged last K-step gets the k rows past the end of its A tile cleared
+    // once it has landed, before the MFMA waves are let in
+    int tail_step[NPH], tail_rows[NPH], acc_steps = 0;
+    if constexpr (TAILS) {
+#pragma unroll
+      for (int i = 0; i < NPH; ++i) {
+        acc_steps += ph[i].K / DMA_BK;
+        tail_rows[i] = (ph[i].a.ks && ph[i].K > 0) ? ph[i].a.ktail : 0;
+        tail_step[i] = acc_steps - 1;
+      }
+    }
     for (int kt = 0; kt < total; ++kt) {
       if (kt + STAGES - 2 < total) wait_vmcnt<AHEAD>();
       else wait_vmcnt<0>();
+      if constexpr (TAILS) {
+#pragma unroll
+        for (int i = 0; i < NPH; ++i)
+          if (tail_rows[i] > 0 && kt == tail_step[i]) DmaLane<TS::BM>::clear_tail(smem + (kt % STAGES) * SM::STAGE, lw, tail_rows[i]);
+      }
       __syncthreads();
       if (issued < total) issue_stage();
     }

@@ -654,7 +654,7 @@ struct TokenReduceDmaParams : TokenReduceParams {
 template <class TS>
 __device__ __forceinline__ void token_reduce_dma_block(const TokenReduceDmaParams& p, int lin, char* smem) {
   constexpr int STAGES = row_stages<TS>();
-  using Pipe = DmaPipe<TS, 1, 2, STAGES>;
+  using Pipe = DmaPipe<TS, 1, 2, STAGES, false, true>;
   int split, tile, bz;   // map: (splits, tiles, 3*nb)
   clear_words(p.prep_clear, lin == 0);
   if (!p.map.locate(lin, split, tile, bz)) return;
@@ -674,7 +674,9 @@ __device__ __forceinline__ void token_reduce_dma_block(const TokenReduceDmaParam
     ph[t].b[0].base = reinterpret_cast<const uint16_t*>(tt.B) + ib * tt.bsB + (size_t)k_begin * tt.ldb + n0;
     ph[t].b[0].ld = tt.ldb; ph[t].b[0].rows = job.N - n0; ph[t].b[0].ks = 1;
     ph[t].nb = 1;
-    ph[t].K = t < job.nterms ? klen : 0;
+    // a token count that is not a multiple of 64 ends inside the last K-step of the last split
+    ph[t].K = t < job.nterms ? (klen + DMA_BK - 1) / DMA_BK * DMA_BK : 0;
+    ph[t].a.ktail = ph[t].b[0].ktail = klen % DMA_BK;
   }
   f32x16 acc[1][TS::TM][TS::TN];
   zero_acc<TS>(acc[0]);

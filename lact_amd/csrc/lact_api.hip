@@ -663,8 +663,8 @@ struct Runner {
 
   // The three token-reduction GEMMs of a step.  Returns the number of partial-sum slots written to the scratch
   // buffer (the caller reduces them), or 0 when the result went straight to `add_out` = coeff*add_in + sum.
-  // bf16: whole blocks of 64 tokens run on the asynchronous-copy kernel (straight to add_out when one split
-  // covers them); a ragged tail of fewer than 64 tokens goes through the generic kernel and is added.
+  // bf16, 64 tokens or more: the asynchronous-copy kernel (straight to add_out when one split covers them; a token
+  // count that is not a multiple of 64 ends inside the last K-step, whose surplus rows the loader clears).
   // `prep` (forward update only): d_out / g16 / ss_part / m_prev / mbar of the momentum step; when the whole
   // reduction is one split of the asynchronous-copy kernel, its epilogue does that step and -1 is returned.
   struct PrepFold {
@@ -691,7 +691,7 @@ struct Runner {
     int main_tokens = 0, slots = 0;
     bool direct = false;
     if constexpr (kBf16) {
-      if (tokens >= 64 && d.d % 8 == 0 && d.dh % 8 == 0) main_tokens = tokens / 64 * 64;
+      if (tokens >= 64 && d.d % 8 == 0 && d.dh % 8 == 0) main_tokens = tokens;   // a ragged end is handled inside the last K-step
       if (main_tokens > 0) {
         const bool big = d.d % TS_NS::BM == 0 && d.dh % TS_NS::BM == 0;
         const int tiles = token_reduce_dma_tiles(d.d, d.dh);
@@ -751,7 +751,7 @@ struct Runner {
         if (main_tokens == tokens) return slots;
       }
     }
-    // generic kernel: everything (fp32, or fewer than 64 tokens) or the ragged tail
+    // generic kernel: fp32, or fewer than 64 tokens
     const int rest = tokens - main_tokens;
     for (int i = 0; i < 3; ++i)
       for (int t = 0; t < p.job[i].nterms; ++t) {
