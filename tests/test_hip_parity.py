@@ -149,7 +149,8 @@ def block_causal_pair(C, use_muon, prenorm=False):
     (2, 2 * 96 + 17, 64, 128, 96, True, False), (2, 2 * 96 + 17, 128, 64, 96, True, True),
     (3, 4 * 200, 384, 384, 200, True, False), (1, 100, 64, 64, 128, True, False),
     (2, 2 * 96 + 17, 40, 136, 96, True, False),    # d not a multiple of 64: generic tile kernels, two hidden tiles
-    (2, 2 * 96 + 17, 64, 192, 96, True, False)])   # dh = 128 + 64: a half-valid hidden tile on the asynchronous-copy path
+    (2, 2 * 96 + 17, 64, 192, 96, True, False),    # dh = 128 + 64: a half-valid hidden tile on the asynchronous-copy path
+    (2, 2 * 3200 + 100, 64, 64, 3200, True, False)])   # long chunks, few tiles: token reductions split in two, partial sums
 def test_block_causal_bf16_no_muon(b, L, d, dh, C, mom, prenorm):
     say("block_causal bf16 no muon", b, L, d, dh, C, mom, prenorm)
     inp = problem(b, L, d, dh, 7, torch.bfloat16, momentum=mom)
@@ -170,7 +171,8 @@ def test_block_causal_bf16_no_muon(b, L, d, dh, C, mom, prenorm):
 
 @pytest.mark.parametrize("b,L,d,dh,C,mom,prenorm", [
     (2, 3 * 64 + 5, 64, 64, 64, True, False), (2, 2 * 96 + 17, 64, 128, 96, True, True),
-    (2, 2 * 96 + 17, 128, 64, 96, False, False), (2, 2 * 96 + 17, 40, 136, 96, True, False)])
+    (2, 2 * 96 + 17, 128, 64, 96, False, False), (2, 2 * 96 + 17, 40, 136, 96, True, False),
+    (2, 2 * 3100 + 50, 64, 64, 3100, True, False)])    # split token reductions on the generic kernels
 def test_block_causal_fp32_no_muon(b, L, d, dh, C, mom, prenorm):
     say("block_causal fp32 no muon", b, L, d, dh, C, mom, prenorm)
     inp = problem(b, L, d, dh, 8, torch.float32, momentum=mom)
