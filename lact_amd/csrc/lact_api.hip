@@ -345,7 +345,7 @@ struct Plan {
     t_xbtmp = sc.take(mat3 * nsz);
     t_ss = sc.take((size_t)3 * d.b * nblk * 4);
     t_dot = sc.take((size_t)3 * d.b * std::max(nblk, 32) * 4);   // partial dots: per chunk of a matrix, or per block of the fused kernel
-    t_mdot = sc.take((size_t)std::max(1, nupd) * 3 * d.b * nblk * 4);   // one slot per update: the momentum gradients are written at the end
+    t_mdot = sc.take((size_t)std::max(1, nupd) * 3 * d.b * std::max(nblk, 256) * 4);   // one slot per update: the momentum gradients are written at the end
     for (int i = 0; i < 2; ++i) t_gwhat[i] = sc.take(mat3 * 4);
     t_gwcur = sc.take(mat3 * 4);
     t_gmcarry = sc.take(mat3 * 4);
@@ -1100,6 +1100,7 @@ struct Runner {
       for (size_t j = i + 1; j < later_updates.size(); ++j)
         if (later_updates[i].start < later_updates[j].end && later_updates[j].start < later_updates[i].end) mg_each = true;
     std::vector<int> mg_updates;
+    int mg_parts = P.nblk;   // partial dots per matrix in a momentum-gradient slot (the same for every update)
     std::vector<std::pair<int, int>> mg_ranges;
     const bool rows_on_side = !seen_q.force && !seen_kv.force && s_side != s_main;
     auto zero_rows = [&](hipStream_t zs) {
@@ -1250,8 +1251,9 @@ struct Runner {
       // momentum state to carry, no raw-gradient term) and every matrix is held as it lies (square shapes).
       const bool dot_in_kernel = ns_all_fused() && P.nsb.size() == 1;
       const bool carry_here = P.momentum && (u > 0 || gm_valid);
-      const bool prep_in_kernel = dot_in_kernel && kBf16 && !carry_here && !(P.muon && d.muon_replaces_weight) &&
+      const bool prep_in_kernel = dot_in_kernel && kBf16 && !(P.muon && d.muon_replaces_weight) &&
                                   P.g.x_contiguous(0) && P.g.x_contiguous(1) && P.g.x_contiguous(2);
+      const size_t mslot = (size_t)3 * d.b * std::max(P.nblk, 256);   // partial momentum dots of one update
       if (P.muon) {
         if (prep_in_kernel) wait_tail();   // the previous update's dk GEMM reads the gradient copy the fused kernel writes
         for (const NsBatch& B : P.nsb) {
@@ -1272,7 +1274,15 @@ struct Runner {
                 f.g16 = reinterpret_cast<const uint16_t*>(g16(u)) + B.xoff;
                 f.dot_part = scr<float>(P.t_dot);
                 f.norms = norms(u) + B.first;
-                if (prep_in_kernel) f.gc = scr<uint16_t>(P.t_gc) + B.xoff;
+                if (prep_in_kernel) {
+                  f.gc = scr<uint16_t>(P.t_gc) + B.xoff;
+                  if (carry_here) {   // as in k_grad_prep
+                    f.gm_carry = gmcarry; f.carry_valid = gm_valid; f.carry_write = u > 0;
+                    f.m_prev = u > 0 ? dsave(u - 1) : nullptr;
+                    f.mbar = u > 0 ? mbar(u) : nullptr;
+                    f.mdot_part = scr<float>(P.t_mdot) + (size_t)u * mslot;
+                  }
+                }
               }
               launch_ns_fused<true>(f, B);
             }
@@ -1334,28 +1344,28 @@ struct Runner {
         p.m_prev = (P.momentum && u > 0) ? dsave(u - 1) : nullptr;
         p.mbar = (P.momentum && u > 0) ? mbar(u) : nullptr;
         p.gc = scr<T>(P.t_gc);
-        p.mdot_part = scr<float>(P.t_mdot) + (size_t)u * 3 * d.b * P.nblk;
+        p.mdot_part = scr<float>(P.t_mdot) + (size_t)u * mslot;
         if (P.muon && ns_fused_any()) p.poison = ns_error_word();
         LACT_LAUNCH("k_grad_prep", "k_grad_prep", 0.0, (k_grad_prep<T, TN>), dim3(P.nblk, 3 * d.b), dim3(256), s, p);
-        if (P.momentum) {
-          gm_valid = true;
-          // the gradient of the per-token momentum needs these dot products only: written by one launch at the end
-          // (by one launch per update, in this order, when token ranges repeat and their shares add up)
-          if (u > 0) {
-            const bool acc = seen_m.accumulate(st.start, st.end);
-            if (acc || mg_each) {
-              MomentumMeanRanges r1;
-              r1.start[0] = st.start; r1.len[0] = T_;
-              LACT_LAUNCH("k_momentum_grad", "k_momentum_grad", 0.0, k_momentum_grad, dim3(d.b, 1), dim3(256), s, scr<float>(P.t_mdot) + (size_t)u * 3 * d.b * P.nblk,
-                          0LL, P.nblk, d.b, dmom, (long long)d.kv_len, r1, acc ? 1 : 0);
-            } else {
-              mg_updates.push_back(u);
-              mg_ranges.emplace_back(st.start, T_);
-            }
+      }
+      if (P.momentum) {
+        gm_valid = true;
+        // partial momentum dots per matrix: one per block of k_grad_prep, or one per tile of the fused kernel
+        mg_parts = (P.muon && prep_in_kernel) ? ns_fused_nbm(P.nsb[0]) : P.nblk;
+        // the gradient of the per-token momentum needs these dot products only: written by one launch at the end
+        // (by one launch per update, in this order, when token ranges repeat and their shares add up)
+        if (u > 0) {
+          const bool acc = seen_m.accumulate(st.start, st.end);
+          if (acc || mg_each) {
+            MomentumMeanRanges r1;
+            r1.start[0] = st.start; r1.len[0] = T_;
+            LACT_LAUNCH("k_momentum_grad", "k_momentum_grad", 0.0, k_momentum_grad, dim3(d.b, 1), dim3(256), s, scr<float>(P.t_mdot) + (size_t)u * mslot,
+                        0LL, mg_parts, d.b, dmom, (long long)d.kv_len, r1, acc ? 1 : 0);
+          } else {
+            mg_updates.push_back(u);
+            mg_ranges.emplace_back(st.start, T_);
           }
         }
-      } else if (P.momentum) {
-        gm_valid = true;   // nothing was carried (first update of the program): as after the kernel above
       }
       const T* kc = k + (size_t)st.start * d.k_ld;
       const T* vc = v + (size_t)st.start * d.v_ld;
@@ -1452,7 +1462,7 @@ struct Runner {
     }
     if (!mg_updates.empty()) {
       // deferred updates are all updates but the first, met in descending order: slot u - 1 of the launch is update u
-      const size_t slot = (size_t)3 * d.b * P.nblk;
+      const size_t slot = (size_t)3 * d.b * std::max(P.nblk, 256);
       const int total = (int)mg_updates.size();
       for (int i0 = 0; i0 < total; i0 += 256) {
         const int n = std::min(256, total - i0);
@@ -1463,7 +1473,7 @@ struct Runner {
           r.start[i] = mg_ranges[idx].first; r.len[i] = mg_ranges[idx].second;
         }
         LACT_LAUNCH("k_momentum_grad", "k_momentum_grad", 0.0, k_momentum_grad, dim3(d.b, n), dim3(256), s, scr<float>(P.t_mdot) + (size_t)umin * slot,
-                    (long long)slot, P.nblk, d.b, dmom, (long long)d.kv_len, r, 0);
+                    (long long)slot, mg_parts, d.b, dmom, (long long)d.kv_len, r, 0);
       }
     }
     {

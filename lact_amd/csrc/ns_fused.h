@@ -56,6 +56,11 @@ struct NsFusedParams {
   //   gc = G_final / (n + 1e-7) - g16 * <G_final, g16> / (n (n + 1e-7)^2)
   // (the gradient w.r.t. the Newton-Schulz input in the compute type; norms as written by the forward)
   float* dot_part; uint16_t* gc;
+  // with gc and a momentum state in the program: the gradient that arrives at the state after this update is added
+  // (carry_valid), the one for the state before it is written back (carry_write: g * mbar), and the partial dots
+  // <g, M_prev> over this block's tile go to mdot_part[z][member] (m_prev set).  All arrays packed like gc.
+  float* gm_carry; int carry_valid, carry_write;
+  const float* m_prev; const float* mbar; float* mdot_part;
   unsigned* sync;            // [n][32] words, zeroed before the launch: word 0 = arrivals, word 1 = XCC id mask
   unsigned* error;           // set to 1 by a block whose barrier timed out
   long long spin_limit;      // polls a block waits at a barrier before it gives up
@@ -287,17 +292,41 @@ __global__ __launch_bounds__(DMA_THREADS) void k_ns_fused(const NsFusedParams p)
       float c0 = 1.f / (n + 1e-7f);
       const float c1 = n > 0.f ? total / (n * (n + 1e-7f) * (n + 1e-7f)) : 0.f;
       if (__hip_atomic_load(p.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) c0 = __uint_as_float(0x7fc00000u);
+      const float mb = p.mbar ? p.mbar[z % p.nb] : 0.f;
+      float md = 0.f;
 #pragma unroll
       for (int t = 0; t < NG; ++t) {
         const int id = threadIdx.x + t * DMA_THREADS;
         if (id < TS::BM * GR) {
           const size_t o = zo + (size_t)(id / GR) * p.c + (id % GR) * 8;
           const uint32_t w[4] = {gi[t].x, gi[t].y, gi[t].z, gi[t].w};
-          Elem<uint16_t>::store4(p.gc + o, ga[t].x * c0 - __uint_as_float(w[0] << 16) * c1, ga[t].y * c0 - __uint_as_float(w[0] & 0xffff0000u) * c1,
-                                 ga[t].z * c0 - __uint_as_float(w[1] << 16) * c1, ga[t].w * c0 - __uint_as_float(w[1] & 0xffff0000u) * c1);
-          Elem<uint16_t>::store4(p.gc + o + 4, gb[t].x * c0 - __uint_as_float(w[2] << 16) * c1, gb[t].y * c0 - __uint_as_float(w[2] & 0xffff0000u) * c1,
-                                 gb[t].z * c0 - __uint_as_float(w[3] << 16) * c1, gb[t].w * c0 - __uint_as_float(w[3] & 0xffff0000u) * c1);
+          float4 v0 = make_float4(ga[t].x * c0 - __uint_as_float(w[0] << 16) * c1, ga[t].y * c0 - __uint_as_float(w[0] & 0xffff0000u) * c1,
+                                  ga[t].z * c0 - __uint_as_float(w[1] << 16) * c1, ga[t].w * c0 - __uint_as_float(w[1] & 0xffff0000u) * c1);
+          float4 v1 = make_float4(gb[t].x * c0 - __uint_as_float(w[2] << 16) * c1, gb[t].y * c0 - __uint_as_float(w[2] & 0xffff0000u) * c1,
+                                  gb[t].z * c0 - __uint_as_float(w[3] << 16) * c1, gb[t].w * c0 - __uint_as_float(w[3] & 0xffff0000u) * c1);
+          if (p.gm_carry) {
+            if (p.carry_valid) {
+              const float4 a = *reinterpret_cast<const float4*>(p.gm_carry + o), b = *reinterpret_cast<const float4*>(p.gm_carry + o + 4);
+              v0.x += a.x; v0.y += a.y; v0.z += a.z; v0.w += a.w;
+              v1.x += b.x; v1.y += b.y; v1.z += b.z; v1.w += b.w;
+            }
+            if (p.carry_write) {
+              *reinterpret_cast<float4*>(p.gm_carry + o) = make_float4(v0.x * mb, v0.y * mb, v0.z * mb, v0.w * mb);
+              *reinterpret_cast<float4*>(p.gm_carry + o + 4) = make_float4(v1.x * mb, v1.y * mb, v1.z * mb, v1.w * mb);
+            }
+            if (p.m_prev) {
+              const float4 a = *reinterpret_cast<const float4*>(p.m_prev + o), b = *reinterpret_cast<const float4*>(p.m_prev + o + 4);
+              md += v0.x * a.x + v0.y * a.y + v0.z * a.z + v0.w * a.w + v1.x * b.x + v1.y * b.y + v1.z * b.z + v1.w * b.w;
+            }
+          }
+          Elem<uint16_t>::store4(p.gc + o, v0.x, v0.y, v0.z, v0.w);
+          Elem<uint16_t>::store4(p.gc + o + 4, v1.x, v1.y, v1.z, v1.w);
         }
+      }
+      if (p.gm_carry && p.m_prev) {
+        __syncthreads();   // the block sum above may still be read from the same LDS words
+        md = block_sum(md, reinterpret_cast<float*>(smem));
+        if (threadIdx.x == 0) p.mdot_part[(size_t)z * nbm + member] = md;
       }
     }
   }
