@@ -340,7 +340,7 @@ struct Plan {
     Bump sc;
     for (int i = 0; i < 6; ++i) t_h[i] = sc.take((size_t)d.b * Tcap * d.dh * esz);
     t_partial = sc.take((size_t)nsplit_max * mat3 * 4);
-    t_lrpart = sc.take((size_t)3 * lr_slots * d.b * Tcap * 4);
+    t_lrpart = sc.take((size_t)std::max(1, nupd) * 3 * lr_slots * d.b * Tcap * 4);   // one slot per update: reduced by one launch at the end
     for (int i = 0; i < 2; ++i) t_xf[i] = sc.take(mat3 * 4);
     t_xbtmp = sc.take(mat3 * nsz);
     t_ss = sc.take((size_t)3 * d.b * nblk * 4);
@@ -1099,6 +1099,18 @@ struct Runner {
     for (size_t i = 0; i < later_updates.size() && !mg_each; ++i)
       for (size_t j = i + 1; j < later_updates.size(); ++j)
         if (later_updates[i].start < later_updates[j].end && later_updates[j].start < later_updates[i].end) mg_each = true;
+    // learning-rate gradients likewise; every update writes them
+    bool lr_each = seen_kv.force;
+    {
+      std::vector<lact_step_t> ups;
+      for (auto& st : P.live)
+        if (st.kind == LACT_UPDATE) ups.push_back(st);
+      for (size_t i = 0; i < ups.size() && !lr_each; ++i)
+        for (size_t j = i + 1; j < ups.size(); ++j)
+          if (ups[i].start < ups[j].end && ups[j].start < ups[i].end) lr_each = true;
+    }
+    std::vector<std::pair<int, int>> lr_ranges;   // met in descending order of the update index, all updates
+    const size_t lrslot = (size_t)3 * P.lr_slots * d.b * P.Tcap;
     std::vector<int> mg_updates;
     int mg_parts = P.nblk;   // partial dots per matrix in a momentum-gradient slot (the same for every update)
     std::vector<std::pair<int, int>> mg_ranges;
@@ -1379,7 +1391,7 @@ struct Runner {
         hp.lr0 = lr0 + st.start; hp.lr1 = lr1 + st.start; hp.lr2 = lr2 + st.start; hp.bslr = d.kv_len;
         hp.G0 = g0; hp.G1 = g1; hp.G2 = g2;
         hp.O0 = h(0); hp.O1 = h(1); hp.O2 = h(2); hp.O3 = h(3); hp.O4 = h(4); hp.O5 = h(5);
-        hp.lrpart = scr<float>(P.t_lrpart);
+        hp.lrpart = scr<float>(P.t_lrpart) + (size_t)u * lrslot;
         hp.lrpart_stride = (long long)d.b * P.Tcap;
         hp.lrpart_mat_stride = (long long)P.lr_slots * d.b * P.Tcap;
         if (P.keep_pre) {
@@ -1428,10 +1440,17 @@ struct Runner {
         if (use_tail || !kBf16) launch_row_gemm<T, true, 2, EPI_STORE>("update_bwd_dv", p, d.b, s, true);
         rows_job.r2 = p;
       }
-      LACT_LAUNCH("k_lr_reduce", "k_lr_reduce", 0.0, k_lr_reduce, dim3(ceil_div(T_, 256), d.b, 3), dim3(256), s, scr<float>(P.t_lrpart),
-                         (long long)P.lr_slots * d.b * P.Tcap, (long long)d.b * P.Tcap,
-                  lr_parts(), P.Tcap, dlr0, dlr1, dlr2,
-                         (long long)d.kv_len, st.start, T_, acc_kv ? 1 : 0);
+      // learning-rate gradients: row partials of every update kept, one reduction launch at the end (one launch per
+      // update, in this order, when token ranges repeat and their shares add up)
+      if (lr_each) {
+        MomentumMeanRanges r1;
+        r1.start[0] = st.start; r1.len[0] = T_;
+        LACT_LAUNCH("k_lr_reduce", "k_lr_reduce", 0.0, k_lr_reduce, dim3(ceil_div(T_, 256), d.b, 3), dim3(256), s,
+                    scr<float>(P.t_lrpart) + (size_t)u * lrslot, 0LL, (long long)P.lr_slots * d.b * P.Tcap, (long long)d.b * P.Tcap, lr_parts(),
+                    P.Tcap, dlr0, dlr1, dlr2, (long long)d.kv_len, r1, acc_kv ? 1 : 0);
+      } else {
+        lr_ranges.emplace_back(st.start, T_);
+      }
       if (use_tail) {
         s = s_main;
         tail_ev = side->event();
@@ -1459,6 +1478,21 @@ struct Runner {
         }
       }
       --ver;
+    }
+    if (!lr_ranges.empty()) {
+      const int total = (int)lr_ranges.size();   // = updates; entry total - 1 - u belongs to update u
+      for (int u0 = 0; u0 < total; u0 += 256) {
+        const int n = std::min(256, total - u0);
+        MomentumMeanRanges r;
+        int longest = 0;
+        for (int i = 0; i < n; ++i) {
+          r.start[i] = lr_ranges[total - 1 - (u0 + i)].first; r.len[i] = lr_ranges[total - 1 - (u0 + i)].second;
+          longest = std::max(longest, r.len[i]);
+        }
+        LACT_LAUNCH("k_lr_reduce", "k_lr_reduce", 0.0, k_lr_reduce, dim3(ceil_div(longest, 256), d.b, 3 * n), dim3(256), s,
+                    scr<float>(P.t_lrpart) + (size_t)u0 * lrslot, (long long)lrslot, (long long)P.lr_slots * d.b * P.Tcap, (long long)d.b * P.Tcap,
+                    lr_parts(), P.Tcap, dlr0, dlr1, dlr2, (long long)d.kv_len, r, 0);
+      }
     }
     if (!mg_updates.empty()) {
       // deferred updates are all updates but the first, met in descending order: slot u - 1 of the launch is update u

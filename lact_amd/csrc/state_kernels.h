@@ -532,13 +532,17 @@ __global__ void k_reduce_partials(float* out, const float* in_add, float coeff, 
   st4(out + e, v);
 }
 
-// dlr_j[ib, start + t] = (or +=, on rows an earlier step of this call wrote) sum over slots of the row partials
-__global__ void k_lr_reduce(const float* lrpart, long long mat_stride, long long slot_stride, int nslots, int Tcap,
-                            float* dlr0, float* dlr1, float* dlr2, long long bs, int start, int len, int accumulate) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x, ib = blockIdx.y, j = blockIdx.z;
+// dlr_j[ib, start + t] = (or +=, on rows an earlier step of this call wrote) sum over slots of the row partials.
+// Grid (ceil(longest chunk / 256), batch, 3 * updates): update i of the launch has its partials at
+// lrpart + i * upd_stride and the token range r[i]; the ranges of one launch do not overlap.
+__global__ void k_lr_reduce(const float* lrpart, long long upd_stride, long long mat_stride, long long slot_stride, int nslots, int Tcap,
+                            float* dlr0, float* dlr1, float* dlr2, long long bs, const MomentumMeanRanges r, int accumulate) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x, ib = blockIdx.y, j = blockIdx.z % 3, i = blockIdx.z / 3;
+  const int start = r.start[i], len = r.len[i];
   if (t >= len) return;
+  const float* part = lrpart + i * upd_stride;
   float s = 0.f;
-  for (int i = 0; i < nslots; ++i) s += lrpart[j * mat_stride + i * slot_stride + (size_t)ib * Tcap + t];
+  for (int k = 0; k < nslots; ++k) s += part[j * mat_stride + k * slot_stride + (size_t)ib * Tcap + t];
   float* dst = j == 0 ? dlr0 : (j == 1 ? dlr1 : dlr2);
   dst += ib * bs + start + t;
   *dst = accumulate ? *dst + s : s;
