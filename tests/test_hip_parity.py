@@ -619,6 +619,19 @@ def test_output_rows_written_twice_belong_to_the_later_apply(act):
     assert max(errs.values()) < (1e-4 if act == torch.float32 else 1e-2)
 
 
+def test_program_with_more_than_256_updates():
+    """Per-update quantities that are written by one launch for the whole program (momentum means, momentum and
+    learning-rate gradients) go in batches of 256 updates: 300 chunks of 64 tokens, fp32 against the oracle."""
+    say("300 updates")
+    b, d, dh, C = 1, 64, 64, 64
+    L = 300 * C + 20
+    inp = problem(b, L, d, dh, 61, torch.float32, momentum=True, lr_shift=-4.0)
+    res, ref = run_both(*block_causal_pair(C, False), inp, PLAIN)
+    errs = compare(res, ref)
+    say("  ", errs)
+    assert max(errs.values()) < 1e-4
+
+
 # ---- size-independent properties at the benchmark size ----------------------------------------------
 def full_size_properties(b, L, d, dh, C, seed, single_update):
     inp = O.make_inputs(b, L, d, dh, seed=seed, act_dtype=torch.bfloat16, distinct_heads=4)
