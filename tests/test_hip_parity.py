@@ -632,6 +632,101 @@ def test_program_with_more_than_256_updates():
     assert max(errs.values()) < 1e-4
 
 
+def _random_program(rng, L):
+    """2 to 7 steps with arbitrary (also overlapping, also repeated) token ranges; at least one apply at the end."""
+    steps = []
+    for _ in range(int(rng.integers(2, 8))):
+        a = int(rng.integers(0, L - 8))
+        e = int(rng.integers(a + 4, min(L, a + 200) + 1))
+        kind = LACT_APPLY if rng.random() < 0.45 else ops.LACT_UPDATE
+        steps.append((kind, a, e, a if kind == LACT_APPLY else 0))
+    a = int(rng.integers(0, L // 2))
+    steps.append((LACT_APPLY, a, L, a))
+    return tuple(steps)
+
+
+@pytest.mark.parametrize("seed", list(range(20)))
+def test_random_programs_match_oracle(seed):
+    """Differential test over random valid programs (random shapes, step lists with overlapping and repeated ranges,
+    momentum / pre-norm / weight-norm / Muon switches): forward and every gradient against the oracle.  fp32
+    activations; Newton-Schulz in fp32 against float64 arithmetic (1e-3), everything else at the fp32 bound 1e-4."""
+    rng = np.random.default_rng(1000 + seed)
+    b = int(rng.integers(1, 3))
+    d = int(rng.choice([16, 40, 64, 128]))
+    dh = int(rng.choice([24, 64, 128, 192]))
+    L = int(rng.integers(60, 400))
+    momentum, prenorm, weight_norm = bool(rng.random() < 0.6), bool(rng.random() < 0.3), bool(rng.random() < 0.8)
+    muon = bool(rng.random() < 0.4)
+    steps = _random_program(rng, L)
+    say("random program", seed, dict(b=b, d=d, dh=dh, L=L, momentum=momentum, prenorm=prenorm, weight_norm=weight_norm, muon=muon), steps)
+    inp = problem(b, L, d, dh, 2000 + seed, torch.float32, momentum=momentum, lr_shift=-2.0)
+    coeffs = O.ns_coeff_table("llm", 5) if muon else None
+    prog = ops.Program(steps=steps, out_len=L, ns_coeffs=coeffs, prenorm=prenorm, weight_norm=weight_norm, ns_mode=ops.NS_FP32)
+    osteps = [O.Step(O.APPLY if k == LACT_APPLY else O.UPDATE, s0, e0) for k, s0, e0, _ in steps]
+
+    def hip(t):
+        return ops.run_program(prog, *args9(t), t["momentum"])[0]
+
+    def orc(t, num):
+        return O.run_program(*args9(t), osteps, num=num, ns_coeffs=coeffs, momentum=t["momentum"], prenorm=prenorm,
+                             weight_norm=weight_norm)[0]
+    g = clone_to(inp, DEV)
+    out = hip(g)
+    go = torch.randn(out.shape, generator=torch.Generator().manual_seed(3))
+    res = {"out": out, **grads_of(out, g, go.to(DEV))}
+    torch.cuda.synchronize()
+    if muon:
+        c = clone_to(inp, "cpu", dtype_map=lambda t: torch.float64)
+        o = orc(c, EXACT)
+        ref = {"out": o, **grads_of(o, c, go.double())}
+        tol = 1e-3
+    else:
+        c = clone_to(inp, "cpu")
+        o = orc(c, PLAIN)
+        ref = {"out": o, **grads_of(o, c, go)}
+        tol = 1e-4
+    errs = compare(res, ref)
+    say("  ", {n: float("%.2e" % e) for n, e in errs.items()})
+    assert max(errs.values()) < tol
+
+
+@pytest.mark.parametrize("seed", list(range(12)))
+def test_random_programs_match_oracle_bf16(seed):
+    """The same differential test on the bf16 path (asynchronous-copy kernels: d, dh multiples of 64; longer
+    ranges), Muon off so that the north-star bound 1e-2 applies outright; the momentum gradient (one dot product per
+    head and chunk) is held to the oracle's own distance from float64 where that distance is large."""
+    rng = np.random.default_rng(5000 + seed)
+    b = int(rng.integers(1, 4))
+    d = int(rng.choice([64, 128, 192]))
+    dh = int(rng.choice([64, 128, 256]))
+    L = int(rng.integers(200, 900))
+    momentum, prenorm, weight_norm = bool(rng.random() < 0.6), bool(rng.random() < 0.3), bool(rng.random() < 0.8)
+    steps = []
+    for _ in range(int(rng.integers(2, 7))):
+        a = int(rng.integers(0, L - 70))
+        e = int(rng.integers(a + 64, min(L, a + 600) + 1))
+        kind = LACT_APPLY if rng.random() < 0.45 else ops.LACT_UPDATE
+        steps.append((kind, a, e, a if kind == LACT_APPLY else 0))
+    a = int(rng.integers(0, L // 2))
+    steps.append((LACT_APPLY, a, L, a))
+    steps = tuple(steps)
+    say("random bf16 program", seed, dict(b=b, d=d, dh=dh, L=L, momentum=momentum, prenorm=prenorm, weight_norm=weight_norm), steps)
+    inp = problem(b, L, d, dh, 6000 + seed, torch.bfloat16, momentum=momentum, lr_shift=-3.0)
+    prog = ops.Program(steps=steps, out_len=L, prenorm=prenorm, weight_norm=weight_norm)
+    osteps = [O.Step(O.APPLY if k == LACT_APPLY else O.UPDATE, s0, e0) for k, s0, e0, _ in steps]
+    hip = lambda t: ops.run_program(prog, *args9(t), t["momentum"])[0]
+    orc = lambda t, num: O.run_program(*args9(t), osteps, num=num, momentum=t["momentum"], prenorm=prenorm, weight_norm=weight_norm)[0]
+    res, ref, r64 = run_both(hip, orc, inp, AC, ref64=True)
+    errs = compare(res, ref)
+    say("  ", {n: float("%.2e" % e) for n, e in errs.items()})
+    for n, e in errs.items():
+        floor = O.rel_l2(ref[n], r64[n])
+        if n == "momentum" and floor > 5e-3:
+            assert O.rel_l2(res[n], r64[n]) <= 1.5 * floor + 2e-3
+        else:
+            assert e < 1e-2, n
+
+
 # ---- size-independent properties at the benchmark size ----------------------------------------------
 def full_size_properties(b, L, d, dh, C, seed, single_update):
     inp = O.make_inputs(b, L, d, dh, seed=seed, act_dtype=torch.bfloat16, distinct_heads=4)
