@@ -24,7 +24,7 @@ def _ar_steps(seq_len, q_len, mini_batch_size, update_length, update_every, num_
     if update_every == -1:
         update_every = mini_batch_size * 2
     first = update_every - mini_batch_size
-    steps = [(LACT_APPLY, 0, first, 0)]
+    steps = [(LACT_APPLY, 0, min(first, q_len), 0)]
     for _ in range(num_repeat):
         for s in range(first, update_length, update_every):
             steps.append((LACT_UPDATE, s, min(s + mini_batch_size, seq_len), 0))   # slices stop at the end (:79-82)

@@ -105,10 +105,26 @@ def test_schedule_builder_matches_oracle(L, C):
 
 
 def test_ar_video_schedule_matches_oracle():
+    """The video step lists against the oracle's, which the oracle tests pin against the reference's loop bounds: the
+    documented case and 300 random argument sets (defaults by -1, cut last windows, updates that stop early,
+    repeats).  The oracle slices tensors (a range past the end is cut there); the builder states the cut ranges."""
+    import numpy as np
     from lact_amd import ar_video
-    mine = ar_video._ar_steps(60, 60, 10, 60, 20, 2)
-    ref = O.ar_video_steps(60, 10, 60, 20, 2)
-    assert [(s[0], s[1], s[2]) for s in mine] == [(0 if s.kind == O.UPDATE else 1, s.start, s.end) for s in ref]
+    cases = [(60, 10, 60, 20, 2)]
+    rng = np.random.default_rng(7)
+    for _ in range(300):
+        L = int(rng.integers(8, 400))
+        mb = int(rng.choice([-1, int(rng.integers(1, L + 1))]))
+        ul = int(rng.choice([-1, int(rng.integers(1, L + 1))]))
+        eff_mb = (L if ul == -1 else ul) if mb == -1 else mb
+        ue = int(rng.choice([-1, eff_mb + int(rng.integers(1, L + 40))]))      # the first window may exceed the sequence
+        cases.append((L, mb, ul, ue, int(rng.integers(1, 4))))
+    for L, mb, ul, ue, rep in cases:
+        mine = ar_video._ar_steps(L, L, mb, ul, ue, rep)
+        ref = O.ar_video_steps(L, mb, ul, ue, rep)
+        cut = [(0 if s.kind == O.UPDATE else 1, min(s.start, L), min(s.end, L)) for s in ref]
+        assert [(s[0], s[1], s[2]) for s in mine] == cut, (L, mb, ul, ue, rep)
+        assert all(s[2] > s[1] for s in mine), (L, mb, ul, ue, rep)      # no empty range reaches the library
 
 
 def test_cpu_tensors_are_refused():
