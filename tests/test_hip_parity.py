@@ -959,7 +959,8 @@ def test_stream_overlap_is_bit_identical(prenorm):
     assert torch.equal(on[0][0], on[2][0]) and all(torch.equal(on[0][1][n], on[2][1][n]) for n in on[0][1])
 
 
-@pytest.mark.parametrize("b,d,dh", [(5, 384, 192), (2, 384, 384), (3, 256, 128)])
+@pytest.mark.parametrize("b,d,dh", [(5, 384, 192), (2, 384, 384), (3, 256, 128),
+                                    (2, 768, 1536)])   # the video model's head: 32 blocks per matrix, a whole XCD per group
 def test_fused_newton_schulz_is_bit_identical(b, d, dh):
     """All Newton-Schulz iterations of an update as one kernel with per-matrix barriers (rows, columns multiples
     of 192) against three GEMM launches per iteration: same tile code, same order, so the same bits in the forward
