@@ -1520,7 +1520,7 @@ struct Runner {
       p.gn0 = gn0; p.n0 = n0(); p.w_init = wf(0);
       p.through_norms = d.detach_norms ? 0 : 1;
       p.out[0] = dw0; p.out[1] = dw1; p.out[2] = dw2;
-      LACT_LAUNCH("k_finish_weight_grads", "k_finish_weight_grads", 0.0, k_finish_weight_grads, rowgrid, dim3(256), s, p);
+      LACT_LAUNCH("k_finish_weight_grads", "k_finish_weight_grads", 0.0, k_finish_weight_grads, eg, dim3(256), s, p);
     }
     LACT_CHECK_LAUNCH();
     return 0;

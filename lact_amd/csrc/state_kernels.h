@@ -556,33 +556,28 @@ struct FinishParams {
   float* out[3];
 };
 __global__ void k_finish_weight_grads(const FinishParams p) {
+  // flat over a matrix, 4 consecutive elements per thread (a row holds a multiple of 4): every lane works
   const int z = blockIdx.y, j = z / p.g.nb, ib = z % p.g.nb;
-  const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-  if (row >= p.g.rows(j)) return;
-  const int cols = p.g.cols(j);
-  const size_t o = (size_t)z * p.g.elems + (size_t)row * cols;
-  float c = 0.f;
+  const long long e = ((long long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (e >= p.g.elems) return;
+  const int cols = p.g.cols(j), row = (int)(e / cols);
+  const size_t o = (size_t)z * p.g.elems + e;
+  float4 v = p.gw ? ld4(p.gw + o) : f4(0.f, 0.f, 0.f, 0.f);
+  if (p.gw2) {
+    const float4 t = ld4(p.gw2 + o);
+    v.x += t.x; v.y += t.y; v.z += t.z; v.w += t.w;
+  }
+  if (p.carry) {
+    const float4 t = ld4(p.carry + o);
+    v.x += t.x; v.y += t.y; v.z += t.z; v.w += t.w;
+  }
   if (p.through_norms) {
     const float n = p.n0[(size_t)z * p.g.maxrows() + row];
-    c = n > 0.f ? p.gn0[(size_t)z * p.g.maxrows() + row] / n : 0.f;
+    const float c = n > 0.f ? p.gn0[(size_t)z * p.g.maxrows() + row] / n : 0.f;
+    const float4 w = ld4(p.w_init + o);
+    v.x += c * w.x; v.y += c * w.y; v.z += c * w.z; v.w += c * w.w;
   }
-  float* dst = p.out[j] + (size_t)ib * p.g.elems + (size_t)row * cols;
-  for (int k = lane * 4; k < cols; k += 256) {
-    float4 v = p.gw ? ld4(p.gw + o + k) : f4(0.f, 0.f, 0.f, 0.f);
-    if (p.gw2) {
-      const float4 t = ld4(p.gw2 + o + k);
-      v.x += t.x; v.y += t.y; v.z += t.z; v.w += t.w;
-    }
-    if (p.carry) {
-      const float4 t = ld4(p.carry + o + k);
-      v.x += t.x; v.y += t.y; v.z += t.z; v.w += t.w;
-    }
-    if (p.through_norms) {
-      const float4 w = ld4(p.w_init + o + k);
-      v.x += c * w.x; v.y += c * w.y; v.z += c * w.z; v.w += c * w.w;
-    }
-    st4(dst + k, v);
-  }
+  st4(p.out[j] + (size_t)ib * p.g.elems + e, v);
 }
 
 // [3b][elems] <-> the three caller tensors, 4 elements per thread
