@@ -972,7 +972,9 @@ struct Runner {
       {
         RenormParams p = renorm_params(u, ver);
         p.main_out = d.prenorm ? main_(u + 1) : nullptr;
-        p.wf_out = wf(ver + 1);
+        // the fp32 copy of a weight version is the base of the next update (and of its backward): the last one has none
+        // (with fp32 activations it is also what the apply steps read)
+        p.wf_out = (P.bf16 && u + 1 == P.nupd) ? nullptr : wf(ver + 1);
         p.wc_out = P.bf16 ? (void*)wc(ver + 1) : nullptr;
         if (u + 1 == P.nupd && w_out)
           for (int j = 0; j < 3; ++j) p.w_ext[j] = w_out[j];

@@ -229,7 +229,7 @@ struct RenormParams {
   int u_stacked;                   // `u` is laid out per Newton-Schulz matrix (MatGeom::u_off), not packed
   int eps_in_sqrt;                 // y = w_hat / sqrt(|w_hat|^2 + eps) * n0 (fused-kernel variant) instead of / (|w_hat| + eps)
   float* main_out;                 // un-normalised accumulator (pre-norm) or null
-  float* wf_out; void* wc_out;     // new weights: fp32 state and compute-type copy (may be null)
+  float* wf_out; void* wc_out;     // new weights: fp32 state and compute-type copy (each may be null)
   float* w_ext[3];                 // caller's weight outputs [b][elems] (same values as wf_out), each nullable
   const unsigned* poison;          // nonzero word: an earlier kernel of this step failed (barrier timeout) -> results become NaN
   // backward only
@@ -297,7 +297,7 @@ __global__ void k_update_renorm(const RenormParams p) {
     // same operation order as the reference: (w / (norm + eps)) * w_norm
     const float4 y = p.weight_norm ? f4((v.x / den) * n0, (v.y / den) * n0, (v.z / den) * n0, (v.w / den) * n0)
                                    : f4(v.x + 0.f * den, v.y + 0.f * den, v.z + 0.f * den, v.w + 0.f * den);
-    st4(p.wf_out + o + c, y);
+    if (p.wf_out) st4(p.wf_out + o + c, y);
     if (ext) st4(ext + c, y);
     if (p.wc_out) Elem<T>::store4(reinterpret_cast<T*>(p.wc_out) + o + c, y.x, y.y, y.z, y.w);
   };
