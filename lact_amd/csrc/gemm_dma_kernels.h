@@ -726,7 +726,7 @@ __device__ __forceinline__ void token_reduce_dma_block(const TokenReduceDmaParam
           float4 v = __builtin_bit_cast(float4, vg[ps % 8]);
           v = make_float4(round_bf16(v.x), round_bf16(v.y), round_bf16(v.z), round_bf16(v.w));
           if (p.prep_m_prev) { v.x += x4[ps].x * mb; v.y += x4[ps].y * mb; v.z += x4[ps].z * mb; v.w += x4[ps].w * mb; }
-          *reinterpret_cast<float4*>(p.prep_d_out + e0 + ps * rstep) = v;
+          if (!p.prep_skip_d) *reinterpret_cast<float4*>(p.prep_d_out + e0 + ps * rstep) = v;
           if (ext) *reinterpret_cast<float4*>(ext + ps * rstep) = v;
           const float f0 = round_bf16(v.x), f1 = round_bf16(v.y), f2 = round_bf16(v.z), f3 = round_bf16(v.w);
           Elem<uint16_t>::store4(p.prep_g16 + e0 + ps * rstep, f0, f1, f2, f3);

@@ -351,6 +351,7 @@ struct TokenReduceParams {
   // layout, and the sum of squares of that copy per block in ss_part[matrix][tile]
   float* prep_d_out; const float* prep_m_prev; const float* prep_mbar; uint16_t* prep_g16; float* prep_ss_part;
   float* prep_m_ext[3];    // caller's momentum outputs [b][elems] per matrix kind (same values as d_out), each nullable
+  int prep_skip_d;         // nothing reads d_out after this update (it stays the switch of the folded epilogue): not stored
   ClearWords prep_clear;   // barrier lines of the fused Newton-Schulz kernel that follows (cleared by the first block)
 };
 

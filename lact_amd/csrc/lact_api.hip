@@ -672,6 +672,7 @@ struct Runner {
   // reduction is one split of the asynchronous-copy kernel, its epilogue does that step and -1 is returned.
   struct PrepFold {
     float* d_out; const float* m_prev; const float* mbar; uint16_t* g16; float* ss_part;
+    bool skip_d;
     float* m_ext[3];
     ClearWords clear;
   };
@@ -708,7 +709,7 @@ struct Runner {
         direct = add_out && sp.n == 1;
         const bool folded = prep && sp.n == 1 && main_tokens == tokens;
         if (folded) {
-          pd.prep_d_out = prep->d_out; pd.prep_m_prev = prep->m_prev; pd.prep_mbar = prep->mbar;
+          pd.prep_d_out = prep->d_out; pd.prep_m_prev = prep->m_prev; pd.prep_mbar = prep->mbar; pd.prep_skip_d = prep->skip_d ? 1 : 0;
           pd.prep_g16 = prep->g16; pd.prep_ss_part = prep->ss_part; pd.prep_clear = prep->clear;
           for (int j = 0; j < 3; ++j) pd.prep_m_ext[j] = prep->m_ext[j];
         } else if (direct) { pd.add_out = add_out; pd.add_in = coeff != 0.f ? add_in : nullptr; pd.coeff = coeff; }
@@ -880,6 +881,9 @@ struct Runner {
         launch_hidden(1, hp, ver, T_);
         upd_z[0] = z0; upd_z[1] = z1; upd_z[2] = z2; upd_zbs = zbs;
       }
+      // the pre-Muon gradient (= the momentum state) of the last update: read by nothing when Newton-Schulz output is
+      // what enters the weights (the next update and its backward would read it; the caller gets its own copy)
+      const bool d_unread = P.muon && !d.muon_replaces_weight && u + 1 == P.nupd;
       int dw_slots = 0;
       {
         TokenReduceJob jobs[3];
@@ -894,10 +898,11 @@ struct Runner {
         // square shapes with Muon: the momentum step can ride in the reduction's epilogue (every tile exists for
         // every matrix, and the Newton-Schulz orientation is the packed one)
         PrepFold pf;
+        pf.skip_d = false;
         const bool can_fold = kBf16 && kNsBf16 && P.muon && !P.g.stacked && d.d == d.dh;
         if (can_fold) {
           for (int j = 0; j < 3; ++j) pf.m_ext[j] = (u + 1 == P.nupd && P.momentum && m_out) ? m_out[j] : nullptr;
-          pf.d_out = dsave(u); pf.m_prev = mprev(u);
+          pf.d_out = dsave(u); pf.m_prev = mprev(u); pf.skip_d = d_unread;
           pf.mbar = has_prev(u) ? mbar(u) : nullptr;
           pf.g16 = reinterpret_cast<uint16_t*>(g16(u)); pf.ss_part = scr<float>(P.t_ss);
           pf.clear.ptr = nullptr; pf.clear.n = 0;
@@ -913,7 +918,7 @@ struct Runner {
         p.g = P.g; p.partial = scr<float>(P.t_partial); p.nsplit = dw_slots;
         p.m_prev = mprev(u);
         p.mbar = has_prev(u) ? mbar(u) : nullptr;
-        p.d_out = dsave(u);
+        p.d_out = d_unread ? nullptr : dsave(u);
         p.g16 = P.muon ? g16(u) : nullptr;
         p.ss_part = scr<float>(P.t_ss);
         p.round_partial_bf16 = P.bf16;
@@ -944,7 +949,7 @@ struct Runner {
               f.xf[0] = scr<float>(P.t_xf[0]) + B.xoff; f.xf[1] = scr<float>(P.t_xf[1]) + B.xoff;
               f.xb = xb(u, 0) + B.xoff; f.xb_it_stride = (long long)P.mat3;
               f.ab = ab(u, 0) + B.sqoff; f.bb = bb(u, 0) + B.sqoff; f.sq_it_stride = (long long)sq3();
-              f.xb_last = scr<uint16_t>(P.t_xbtmp) + B.xoff; f.u_out = usave(u) + B.xoff;
+              f.u_out = usave(u) + B.xoff;
               if (scale_in_kernel) {
                 f.g16 = reinterpret_cast<const uint16_t*>(g16(u)) + B.xoff;
                 f.ss_part = scr<float>(P.t_ss); f.nparts = ss_parts;

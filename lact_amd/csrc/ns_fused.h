@@ -43,7 +43,6 @@ struct NsFusedParams {
   float* xf[2];
   uint16_t* xb; long long xb_it_stride;            // X_k at xb + k * xb_it_stride, k < S
   uint16_t* ab; uint16_t* bb; long long sq_it_stride;
-  uint16_t* xb_last;                               // bf16 copy of X_S (scratch)
   float* u_out;                                    // X_S, fp32, original orientation
   // backward: incoming gradient in gxf[0] / gxb[0]; the result ends in gxf[S & 1]
   float* gxf[2]; uint16_t* gxb[2]; uint16_t* sg; uint16_t* gas;
@@ -210,7 +209,7 @@ __global__ __launch_bounds__(DMA_THREADS) void k_ns_fused(const NsFusedParams p)
         q.g.aux = p.xf[it & 1]; q.g.ldaux = c; q.g.bsaux = xe; q.g.alpha = 1.f; q.g.beta = ca;
         q.g.round_out_bf16 = p.plain;
         q.g.out = last ? nullptr : p.xf[(it + 1) & 1];
-        q.g.out_c = last ? p.xb_last : p.xb + (it + 1) * p.xb_it_stride;
+        q.g.out_c = last ? nullptr : p.xb + (it + 1) * p.xb_it_stride;   // nothing multiplies by the last iterate
         q.g.out_t = last ? p.u_out : nullptr;
         q.g.transpose_mask = p.mask; q.g.nb = p.nb;
         row_gemm_tile<TS, 1, EPI_AXPBY_F32_DUAL, true, true>(q, rx, ry, z, smem);

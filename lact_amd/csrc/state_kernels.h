@@ -116,7 +116,7 @@ struct MomentumPrepParams {
   const float* partial; int nsplit;   // [nsplit][3b][elems]
   const float* m_prev;                // [3b][elems] or null (no momentum / first update uses zeros)
   const float* mbar;                  // [b] or null
-  float* d_out;                       // [3b][elems]  dw (+ momentum): new momentum state, pre-Muon gradient
+  float* d_out;                       // [3b][elems]  dw (+ momentum): new momentum state, pre-Muon gradient (null: nothing reads it)
   float* m_ext[3];                    // caller's momentum outputs [b][elems] (same values as d_out), each nullable
   void* g16;                          // [3b][elems]  d_out cast to the Newton-Schulz type, in its orientation, or null
   float* ss_part;                     // [3b][gridDim.x]
@@ -146,7 +146,7 @@ __global__ void k_momentum_prep(const MomentumPrepParams p) {
       const float4 m = ld4(p.m_prev + zo + e);
       v.x += m.x * mb; v.y += m.y * mb; v.z += m.z * mb; v.w += m.w * mb;
     }
-    st4(p.d_out + zo + e, v);
+    if (p.d_out) st4(p.d_out + zo + e, v);
     if (ext) st4(ext + e, v);
     if (p.g16) {
       const float4 f = f4(Elem<TN>::rnd(v.x), Elem<TN>::rnd(v.y), Elem<TN>::rnd(v.z), Elem<TN>::rnd(v.w));
