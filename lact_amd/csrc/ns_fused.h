@@ -248,7 +248,7 @@ __global__ __launch_bounds__(DMA_THREADS) void k_ns_fused(const NsFusedParams p)
         q.g.M = r; q.g.N = c; q.g.ldo = c; q.g.bso = xe;
         q.g.aux = p.gxf[cur]; q.g.ldaux = c; q.g.bsaux = xe; q.g.alpha = 1.f; q.g.beta = ca;
         q.g.out = p.gxf[cur ^ 1];
-        q.g.out_c = p.gxb[cur ^ 1];
+        q.g.out_c = step + 1 == p.S ? nullptr : p.gxb[cur ^ 1];   // nothing multiplies by the final gradient
         row_gemm_tile<TS, 2, EPI_AXPBY_F32_DUAL, true, true>(q, rx, ry, z, smem);
       }
       LACT_NS_TS(1 + step * 6 + 4);
