@@ -38,11 +38,11 @@ CONFIGS = {
 # HBM bytes per launch at config 1 (read + write), from the FETCH_SIZE / WRITE_SIZE counters of two
 # `rocprofv3 --pmc` runs scaled by a 1 GiB copy (profiles/c1_fwd_bwd_hbm_traffic_pmc.txt); MiB.
 MEASURED_TRAFFIC_MIB = {
-    "k_ns_fused<192x192,bwd>": 751.2 + 357.9,
-    "k_ns_fused<192x192,fwd>": 434.9 + 387.1,
-    "k_token_reduce_dma<192x192>": 120.3 + 31.5,
-    "k_token_reduce_rows_dma<192x192>": 353.5 + 75.0,
-    "k_update_bwd_hidden_kept_dma": 151.9 + 74.2,
+    "k_ns_fused<192x192,bwd>": 749.1 + 344.4,
+    "k_ns_fused<192x192,fwd>": 435.2 + 373.6,
+    "k_token_reduce_dma<192x192>": 120.3 + 22.5,
+    "k_token_reduce_rows_dma<192x192>": 355.6 + 75.0,
+    "k_update_bwd_hidden_kept_dma": 151.8 + 74.2,
     "k_apply_bwd_hidden_dma": 77.9 + 72.0,
     "k_update_hidden_dma": 79.1 + 144.0,
     "k_apply_hidden_dma": 33.2 + 24.0,
@@ -50,7 +50,7 @@ MEASURED_TRAFFIC_MIB = {
 
 
 # Whole step at config 1, same two counter runs (last line of that profile): read + written MiB
-MEASURED_STEP_TRAFFIC_MIB = 2792.0 + 1646.0
+MEASURED_STEP_TRAFFIC_MIB = 2792.0 + 1565.0
 PEAK_HBM_GBPS = 8000.0
 
 
