@@ -89,6 +89,7 @@ __device__ __forceinline__ void row_gemm_tile(const RowGemmDmaParams<NT>& pp, in
         }
       }
       const float al = EPI == EPI_STORE ? 1.f : p.alpha, be = EPI == EPI_STORE ? 1.f : p.beta;
+      uint16_t* dst2 = (EPI == EPI_STORE && p.out2) ? reinterpret_cast<uint16_t*>(p.out2) + (dst - reinterpret_cast<uint16_t*>(p.out)) : nullptr;
       // LDS reads in unconditional groups of 8 (a branch per row would put every read's latency in line)
       uint4 ug[8];
 #pragma unroll
@@ -102,18 +103,28 @@ __device__ __forceinline__ void row_gemm_tile(const RowGemmDmaParams<NT>& pp, in
         if (r < TS::BM && m0 + r < p.M) {
           uint4 u = ug[ps % 8];
           if (blend) {
+            // the staged values are round(acc); each product and the sum are tensors of their own in the reference
             uint32_t uu[4] = {u.x, u.y, u.z, u.w}, ww[4] = {w[ps].x, w[ps].y, w[ps].z, w[ps].w};
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-              const float lo = al * __uint_as_float(uu[j] << 16) + be * __uint_as_float(ww[j] << 16);
-              const float hi = al * __uint_as_float(uu[j] & 0xffff0000u) + be * __uint_as_float(ww[j] & 0xffff0000u);
+              const float lo = round_bf16(al * __uint_as_float(uu[j] << 16)) + round_bf16(be * __uint_as_float(ww[j] << 16));
+              const float hi = round_bf16(al * __uint_as_float(uu[j] & 0xffff0000u)) + round_bf16(be * __uint_as_float(ww[j] & 0xffff0000u));
               uu[j] = (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
             }
             u = make_uint4(uu[0], uu[1], uu[2], uu[3]);
           }
           *reinterpret_cast<uint4*>(dst) = u;
+          if (dst2) {
+            uint32_t uu[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              uu[j] = (uint32_t)f32_to_bf16(p.alpha2 * __uint_as_float(uu[j] << 16)) |
+                      ((uint32_t)f32_to_bf16(p.alpha2 * __uint_as_float(uu[j] & 0xffff0000u)) << 16);
+            *reinterpret_cast<uint4*>(dst2) = make_uint4(uu[0], uu[1], uu[2], uu[3]);
+          }
         }
         dst += dstep;
+        if (dst2) dst2 += dstep;
       }
     }
   } else {
@@ -149,12 +160,11 @@ __device__ __forceinline__ void row_gemm_tile(const RowGemmDmaParams<NT>& pp, in
         if (r < TS::BM && m0 + r < p.M) {
           float4* sp = reinterpret_cast<float4*>(src + ps * ST::RPP * ST::LD * 4);
           const float4 a4 = __builtin_bit_cast(float4, ag[ps % 8]);
-          float v[4] = {p.alpha * a4.x + p.beta * x4[ps].x, p.alpha * a4.y + p.beta * x4[ps].y, p.alpha * a4.z + p.beta * x4[ps].z,
-                        p.alpha * a4.w + p.beta * x4[ps].w};
-          if (p.round_out_bf16) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) v[j] = round_bf16(v[j]);
-          }
+          // the matrix product is a bf16 tensor in the reference (ttt_operation.py:62)
+          float v[4] = {dual_blend(__fmul_rn(p.alpha, round_bf16(a4.x)), __fmul_rn(p.beta, x4[ps].x), p.round_out_bf16),
+                        dual_blend(__fmul_rn(p.alpha, round_bf16(a4.y)), __fmul_rn(p.beta, x4[ps].y), p.round_out_bf16),
+                        dual_blend(__fmul_rn(p.alpha, round_bf16(a4.z)), __fmul_rn(p.beta, x4[ps].z), p.round_out_bf16),
+                        dual_blend(__fmul_rn(p.alpha, round_bf16(a4.w)), __fmul_rn(p.beta, x4[ps].w), p.round_out_bf16)};
           if (p.out) Elem<float>::store4(reinterpret_cast<float*>(p.out) + off, v[0], v[1], v[2], v[3]);
           if (p.out_c) Elem<uint16_t>::store4(reinterpret_cast<uint16_t*>(p.out_c) + off, v[0], v[1], v[2], v[3]);
           if (p.out_t && !tr) Elem<float>::store4(p.out_t + off, v[0], v[1], v[2], v[3]);
@@ -319,6 +329,9 @@ __device__ __forceinline__ void three_acc_mainloop(const HiddenDmaParams& pp, ch
   __syncthreads();
 }
 
+// update forward.  O0 = dgate_before_act, O1 = hidden * lr1, O2 = dhidden_before_mul (the operands of the three
+// fast-weight gradient GEMMs: lr0 and lr2 scale k there, ttt_operation.py:166-168).  For the backward, when O3 is set:
+// O3..O5 = the rounded pre-activations, O6 = O0 * lr0, O7 = O2 * lr2.  Staged four tiles at a time.
 template <class TS>
 __global__ __launch_bounds__(DMA_THREADS) void k_update_hidden_dma(const HiddenDmaParams pp) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -329,8 +342,10 @@ __global__ __launch_bounds__(DMA_THREADS) void k_update_hidden_dma(const HiddenD
   f32x16 a02[2][TS::TM][TS::TN], a1[1][TS::TM][TS::TN];
   three_acc_mainloop<TS>(pp, smem, m0, n0, z, a02, a1);
   using SB = StageTile<TS, 2>;
-  char* s0 = smem + SB::lane_base(); char* s1 = s0 + SB::BYTES; char* s2 = s0 + 2 * SB::BYTES;
-  const int ntm = threadIdx.x < TS::THREADS ? TS::TM : 0;   // the loader wave owns no fragments
+  char* s0 = smem + SB::lane_base(); char* s1 = s0 + SB::BYTES; char* s2 = s0 + 2 * SB::BYTES; char* s3 = s0 + 3 * SB::BYTES;
+  const int ntm = threadIdx.x < TS::THREADS ? TS::TM : 0;   // the loader waves own no fragments
+  const bool keep = p.O3 != nullptr;
+  uint32_t z2p[TS::TM][TS::TN][8];   // O7 waits for the second round, packed in pairs
 #pragma unroll
   for (int tm = 0; tm < TS::TM; ++tm) {
     if (tm >= ntm) break;
@@ -342,17 +357,23 @@ __global__ __launch_bounds__(DMA_THREADS) void k_update_hidden_dma(const HiddenD
     for (int tn = 0; tn < TS::TN; ++tn)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        float z0[4], z1[4], z2[4];
+        float z0[4], z1[4], z2[4], y0[4], y2[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const float gg = round_bf16(a02[0][tm][tn][4 * g + j]), h2 = round_bf16(a02[1][tm][tn][4 * g + j]);
           const float dh = round_bf16(a1[0][tm][tn][4 * g + j]);
           const UpdatePointwise u = update_pointwise<uint16_t>(gg, h2, dh, silu_parts(gg));
-          z0[j] = u.dgpre * l0; z1[j] = u.hid * l1; z2[j] = u.dh2 * l2;
+          z0[j] = u.dgpre; z1[j] = u.hid * l1; z2[j] = u.dh2;
+          y0[j] = u.dgpre * l0; y2[j] = u.dh2 * l2;
         }
         SB::put4(s0, tm, tn, g, z0[0], z0[1], z0[2], z0[3]);
         SB::put4(s1, tm, tn, g, z1[0], z1[1], z1[2], z1[3]);
         SB::put4(s2, tm, tn, g, z2[0], z2[1], z2[2], z2[3]);
+        if (keep) {
+          SB::put4(s3, tm, tn, g, y0[0], y0[1], y0[2], y0[3]);
+          z2p[tm][tn][2 * g] = (uint32_t)f32_to_bf16(y2[0]) | ((uint32_t)f32_to_bf16(y2[1]) << 16);
+          z2p[tm][tn][2 * g + 1] = (uint32_t)f32_to_bf16(y2[2]) | ((uint32_t)f32_to_bf16(y2[3]) << 16);
+        }
       }
   }
   __syncthreads();
@@ -360,7 +381,8 @@ __global__ __launch_bounds__(DMA_THREADS) void k_update_hidden_dma(const HiddenD
   copy_out_b16<TS>(smem + 0 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O0) + off, p.dh, p.T - m0, p.dh - n0);
   copy_out_b16<TS>(smem + 1 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O1) + off, p.dh, p.T - m0, p.dh - n0);
   copy_out_b16<TS>(smem + 2 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O2) + off, p.dh, p.T - m0, p.dh - n0);
-  if (p.O3) {   // the backward is going to start from the rounded pre-activations instead of recomputing them
+  if (keep) {   // the backward is going to start from the rounded pre-activations instead of recomputing them
+    copy_out_b16<TS>(smem + 3 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O6) + off, p.dh, p.T - m0, p.dh - n0);
     __syncthreads();
 #pragma unroll
     for (int tm = 0; tm < TS::TM; ++tm) {
@@ -372,12 +394,14 @@ __global__ __launch_bounds__(DMA_THREADS) void k_update_hidden_dma(const HiddenD
           SB::put4(s0, tm, tn, g, a02[0][tm][tn][4 * g], a02[0][tm][tn][4 * g + 1], a02[0][tm][tn][4 * g + 2], a02[0][tm][tn][4 * g + 3]);
           SB::put4(s1, tm, tn, g, a02[1][tm][tn][4 * g], a02[1][tm][tn][4 * g + 1], a02[1][tm][tn][4 * g + 2], a02[1][tm][tn][4 * g + 3]);
           SB::put4(s2, tm, tn, g, a1[0][tm][tn][4 * g], a1[0][tm][tn][4 * g + 1], a1[0][tm][tn][4 * g + 2], a1[0][tm][tn][4 * g + 3]);
+          *reinterpret_cast<uint2*>(s3 + SB::frag_off(tm, tn, g)) = make_uint2(z2p[tm][tn][2 * g], z2p[tm][tn][2 * g + 1]);
         }
     }
     __syncthreads();
     copy_out_b16<TS>(smem + 0 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O3) + off, p.dh, p.T - m0, p.dh - n0);
     copy_out_b16<TS>(smem + 1 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O4) + off, p.dh, p.T - m0, p.dh - n0);
     copy_out_b16<TS>(smem + 2 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O5) + off, p.dh, p.T - m0, p.dh - n0);
+    copy_out_b16<TS>(smem + 3 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O7) + off, p.dh, p.T - m0, p.dh - n0);
   }
 }
 
@@ -400,7 +424,7 @@ __global__ __launch_bounds__(DMA_THREADS) void k_apply_bwd_hidden_dma(const Hidd
       const float gh = round_bf16(a1[0][tm][tn][4 * g + j]);
       const SiluParts s = silu_parts(y0);
       const float sg = round_bf16(s.silu);
-      hq[j] = sg * y2; gy0[j] = gh * y2 * s.d1; gy2[j] = gh * sg;
+      hq[j] = sg * y2; gy0[j] = round_bf16(gh * y2) * s.d1; gy2[j] = gh * sg;
     }
     SB::put4(s0, tm, tn, g, hq[0], hq[1], hq[2], hq[3]);
     SB::put4(s1, tm, tn, g, gy0[0], gy0[1], gy0[2], gy0[3]);
@@ -725,7 +749,10 @@ __device__ __forceinline__ void token_reduce_dma_block(const TokenReduceDmaParam
         if (r < TS::BM && m0 + r < job.M) {
           float4 v = __builtin_bit_cast(float4, vg[ps % 8]);
           v = make_float4(round_bf16(v.x), round_bf16(v.y), round_bf16(v.z), round_bf16(v.w));
-          if (p.prep_m_prev) { v.x += x4[ps].x * mb; v.y += x4[ps].y * mb; v.z += x4[ps].z * mb; v.w += x4[ps].w * mb; }
+          if (p.prep_m_prev) {   // product and sum rounded separately, as the reference's two tensor operations are
+            v.x = __fadd_rn(v.x, __fmul_rn(x4[ps].x, mb)); v.y = __fadd_rn(v.y, __fmul_rn(x4[ps].y, mb));
+            v.z = __fadd_rn(v.z, __fmul_rn(x4[ps].z, mb)); v.w = __fadd_rn(v.w, __fmul_rn(x4[ps].w, mb));
+          }
           if (!p.prep_skip_d) *reinterpret_cast<float4*>(p.prep_d_out + e0 + ps * rstep) = v;
           if (ext) *reinterpret_cast<float4*>(ext + ps * rstep) = v;
           const float f0 = round_bf16(v.x), f1 = round_bf16(v.y), f2 = round_bf16(v.z), f3 = round_bf16(v.w);

@@ -37,13 +37,25 @@ struct RowGemmParams {
   int M, N;
   void* out; int ldo; long long bso;          // EPI_STORE, EPI_AXPBY: type T; DUAL: fp32
   int accumulate;                              // EPI_STORE only: out += result
-  // out = alpha * round(acc) + beta * aux
+  // EPI_STORE only, optional: out2 = round(alpha2 * round(acc)), type T, laid out like out (the product c*A that
+  // ttt_operation.py:60 forms as a tensor of its own before the matmul)
+  void* out2; float alpha2;
+  // Every value that is a tensor in the reference's eager evaluation is rounded to its type T (identity for fp32):
+  //   EPI_AXPBY:  out = round(round(alpha * round(acc)) + round(beta * aux))           (ttt_operation.py:59-61)
+  //   DUAL:       out = alpha * round(acc) + beta * aux in fp32                        (:62 under autocast)
+  //               round_out_bf16: round(round(alpha * round(acc)) + round(beta * aux)) (:62 without autocast)
   const void* aux; int ldaux; long long bsaux; // EPI_AXPBY: aux of type T; DUAL: fp32 aux
   float alpha, beta;
   void* out_c;                                 // DUAL: copy in type T, same ld/bs as out
   float* out_t; int transpose_mask; int nb;    // DUAL: optional fp32 copy; matrices whose (z / nb) bit is set are written transposed
   int round_out_bf16;                          // DUAL: round the fp32 result to bf16 (reference without autocast)
 };
+
+// X' = a X + B X (ttt_operation.py:62): `prod` = alpha * round(acc), `ax` = beta * aux.  Without autocast both are bf16
+// tensors and so is their sum.
+__device__ __forceinline__ float dual_blend(float prod, float ax, int plain_bf16) {
+  return plain_bf16 ? round_bf16(round_bf16(prod) + round_bf16(ax)) : __fadd_rn(ax, prod);
+}
 
 template <typename T, class TS, bool B_KC, int NT, int EPI>
 __global__ __launch_bounds__(TS::THREADS) void k_row_gemm(const RowGemmParams<NT> p) {
@@ -72,20 +84,22 @@ __global__ __launch_bounds__(TS::THREADS) void k_row_gemm(const RowGemmParams<NT
         for (int j = 0; j < 4; ++j) v[j] += old[j];
       }
       Elem<T>::store4(o, v[0], v[1], v[2], v[3]);
+      if (p.out2) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = p.alpha2 * Elem<T>::rnd(v[j]);
+        Elem<T>::store4(reinterpret_cast<T*>(p.out2) + z * p.bso + (size_t)m * p.ldo + n, v[0], v[1], v[2], v[3]);
+      }
     } else if (EPI == EPI_AXPBY) {
       float a[4];
       Elem<T>::load4(reinterpret_cast<const T*>(p.aux) + z * p.bsaux + (size_t)m * p.ldaux + n, a);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) v[j] = p.alpha * Elem<T>::rnd(v[j]) + p.beta * a[j];
+      for (int j = 0; j < 4; ++j) v[j] = Elem<T>::rnd(p.alpha * Elem<T>::rnd(v[j])) + Elem<T>::rnd(p.beta * a[j]);
       Elem<T>::store4(reinterpret_cast<T*>(p.out) + z * p.bso + (size_t)m * p.ldo + n, v[0], v[1], v[2], v[3]);
     } else {
       float a[4];
       Elem<float>::load4(reinterpret_cast<const float*>(p.aux) + z * p.bsaux + (size_t)m * p.ldaux + n, a);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        v[j] = p.alpha * Elem<T>::rnd(v[j]) + p.beta * a[j];
-        if (p.round_out_bf16) v[j] = round_bf16(v[j]);
-      }
+      for (int j = 0; j < 4; ++j) v[j] = dual_blend(__fmul_rn(p.alpha, Elem<T>::rnd(v[j])), __fmul_rn(p.beta, a[j]), p.round_out_bf16);
       const size_t off = z * p.bso + (size_t)m * p.ldo + n;
       if (p.out) Elem<float>::store4(reinterpret_cast<float*>(p.out) + off, v[0], v[1], v[2], v[3]);
       if (p.out_c) Elem<T>::store4(reinterpret_cast<T*>(p.out_c) + off, v[0], v[1], v[2], v[3]);
@@ -115,6 +129,7 @@ struct HiddenParams {
   // gradients of the fast-weight gradients (backward of the update): G0,G2 [dh,d], G1 [d,dh], type T
   const void* G0; const void* G1; const void* G2;
   void* O0; void* O1; void* O2; void* O3; void* O4; void* O5;  // [b, T, dh] outputs, type T
+  void* O6; void* O7;               // update forward: lr-scaled copies of O0 and O2 kept for the backward (nullable)
   long long bso;
   // update backward from kept pre-activations: I0 = k W0^T, I1 = k W2^T, I2 = v W1 as the forward rounded them
   const void* I0; const void* I1; const void* I2; long long bsi;
@@ -159,12 +174,17 @@ __device__ __forceinline__ UpdatePointwise update_pointwise(float g, float h2, f
   const float sg = Elem<T>::rnd(s.silu);
   u.hid = Elem<T>::rnd(sg * h2);                       // ttt_operation.py:150
   u.dh2 = Elem<T>::rnd(dh * sg);                       // :155
-  u.dgpre = Elem<T>::rnd(Elem<T>::rnd(dh * h2) * s.d1);  // :157-158
+  // silu_backprop(dhidden * hidden_before_mul, gate_before_act), :157-158 with :15-16 evaluated operation by
+  // operation on tensors of type T as eager PyTorch does: dy * sigma * (1 + x * (1 - sigma))
+  const float sb = Elem<T>::rnd(s.sig), dg = Elem<T>::rnd(dh * h2);
+  const float t1 = Elem<T>::rnd(dg * sb);
+  const float t4 = Elem<T>::rnd(1.f + Elem<T>::rnd(g * Elem<T>::rnd(1.f - sb)));
+  u.dgpre = Elem<T>::rnd(t1 * t4);
   return u;
 }
 
-// update forward:  O0 = dgate_before_act * lr0, O1 = hidden * lr1, O2 = dhidden_before_mul * lr2
-// (ttt_operation.py:147-168; the lr is folded into the token-major operand of each reduction GEMM).
+// update forward:  O0 = dgate_before_act, O1 = hidden * lr1, O2 = dhidden_before_mul
+// (ttt_operation.py:147-168: lr1 scales the hidden-side operand of dw1, lr0 and lr2 scale k -- see k_lr_scale_rows).
 template <typename T, class TS>
 __global__ __launch_bounds__(TS::THREADS) void k_update_hidden(const HiddenParams p) {
   __shared__ __attribute__((aligned(16))) char smem[GemmSmem<T, TS>::BYTES];
@@ -184,22 +204,40 @@ __global__ __launch_bounds__(TS::THREADS) void k_update_hidden(const HiddenParam
   LACT_FOR_QUADS(TS) {
     const int m = m0 + quad_m<TS>(tm), n = n0 + quad_n<TS>(tn, g);
     if (m >= p.T || n >= p.dh) continue;
-    const float l0 = p.lr0[z * p.bslr + m], l1 = p.lr1[z * p.bslr + m], l2 = p.lr2[z * p.bslr + m];
+    const float l1 = p.lr1[z * p.bslr + m];
     float z0[4], z1[4], z2[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const float gg = Elem<T>::rnd(a0[tm][tn][4 * g + j]), h2 = Elem<T>::rnd(a2[tm][tn][4 * g + j]);
       const float dh = Elem<T>::rnd(a1[tm][tn][4 * g + j]);
       const UpdatePointwise u = update_pointwise<T>(gg, h2, dh, silu_parts(gg));
-      z0[j] = u.dgpre * l0;
+      z0[j] = u.dgpre;
       z1[j] = u.hid * l1;
-      z2[j] = u.dh2 * l2;
+      z2[j] = u.dh2;
     }
     const size_t off = z * p.bso + (size_t)m * p.dh + n;
     Elem<T>::store4(reinterpret_cast<T*>(p.O0) + off, z0[0], z0[1], z0[2], z0[3]);
     Elem<T>::store4(reinterpret_cast<T*>(p.O1) + off, z1[0], z1[1], z1[2], z1[3]);
     Elem<T>::store4(reinterpret_cast<T*>(p.O2) + off, z2[0], z2[1], z2[2], z2[3]);
   }
+}
+
+// kl0 = T(k * lr0), kl2 = T(k * lr2): the token-major operands of the dw0 and dw2 reductions.  The reference scales
+// k by the per-token rate and casts the product before the matmul (ttt_operation.py:167-168, lact_ttt.py:122-126),
+// so the rounding has to happen on this side of the contraction.  k: [b, tokens, d] with row / batch strides;
+// outputs contiguous [b][tokens][d] with batch stride bso.  Grid (ceil(tokens * d / 4 / 256), b).
+template <typename T>
+__global__ void k_lr_scale_rows(const T* k, int ld, long long bs, const float* lr0, const float* lr2, long long bslr,
+                                int tokens, int d, T* o0, T* o2, long long bso) {
+  const long long e = ((long long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  const int z = blockIdx.y;
+  if (e >= (long long)tokens * d) return;
+  const int t = (int)(e / d), c = (int)(e % d);
+  float v[4];
+  Elem<T>::load4(k + z * bs + (size_t)t * ld + c, v);
+  const float l0 = lr0[z * bslr + t], l2 = lr2[z * bslr + t];
+  Elem<T>::store4(o0 + z * bso + e, v[0] * l0, v[1] * l0, v[2] * l0, v[3] * l0);
+  Elem<T>::store4(o2 + z * bso + e, v[0] * l2, v[1] * l2, v[2] * l2, v[3] * l2);
 }
 
 // Row sums over the hidden dimension of a per-thread partial: lanes l and l^32 hold the same token.
@@ -242,7 +280,7 @@ __global__ __launch_bounds__(TS::THREADS) void k_apply_bwd_hidden(const HiddenPa
       const SiluParts s = silu_parts(y0);
       const float sg = Elem<T>::rnd(s.silu);
       hq[j] = sg * y2;
-      gy0[j] = gh * y2 * s.d1;
+      gy0[j] = Elem<T>::rnd(gh * y2) * s.d1;   // the gradient of the gate is a tensor of type T before silu's backward
       gy2[j] = gh * sg;
     }
     const size_t off = z * p.bso + (size_t)m * p.dh + n;

@@ -205,15 +205,16 @@ struct Plan {
   size_t mat3 = 0;  // 3*b*elems
   // saved
   size_t s_n0, s_wf, s_wc, s_main, s_d, s_min, s_mbar, s_u, s_g16, s_norms, s_xb, s_ab, s_bb, saved_bytes;
-  // Kept for the backward on the asynchronous-copy path: per update, six token-major arrays [b][T][dh] -- the three
-  // lr-scaled operands of the fast-weight gradient GEMMs and the three rounded pre-activations they came from.
+  // Kept for the backward on the asynchronous-copy path: per update, eight token-major arrays [b][T][dh] -- the three
+  // lr-scaled hidden-side operands the backward's GEMMs read, the three rounded pre-activations they came from, and
+  // the two unscaled operands of the forward's dw0 / dw2 reductions (which scale k instead).
   // 288 GB of HBM make keeping them cheaper than the three GEMMs that would recompute them.
   bool keep_pre = false;
   std::vector<size_t> s_pre;   // by update index
   std::vector<int> pre_T;
   // scratch
   size_t t_h[6], t_partial, t_lrpart, t_xf[2], t_xbtmp, t_ss, t_dot, t_mdot, t_gwhat[2], t_gwcur, t_gmcarry, t_gc,
-      t_gxf[2], t_gxb[2], t_sg, t_gas, t_gn0, t_hs[3], t_partial_side, t_gwside[2], t_nssync, scratch_bytes;
+      t_gxf[2], t_gxb[2], t_sg, t_gas, t_gn0, t_hs[3], t_partial_side, t_gwside[2], t_nssync, t_kl[2], t_ca, scratch_bytes;
 
   int build(const lact_desc_t* desc) {
     if (!desc) return fail("null descriptor");
@@ -333,7 +334,7 @@ struct Plan {
       for (const auto& st : steps)
         if (st.kind == LACT_UPDATE) {
           pre_T.push_back(st.end - st.start);
-          s_pre.push_back(sv.take((size_t)6 * d.b * (st.end - st.start) * d.dh * esz));
+          s_pre.push_back(sv.take((size_t)8 * d.b * (st.end - st.start) * d.dh * esz));
         }
     saved_bytes = sv.off + 256;
 
@@ -360,6 +361,8 @@ struct Plan {
     t_partial_side = sc.take((size_t)nsplit_max * mat3 * 4);
     for (int i = 0; i < 2; ++i) t_gwside[i] = sc.take(mat3 * 4);
     t_nssync = sc.take(((size_t)3 * d.b * 32 + 32) * 4);   // per-matrix barrier lines of the fused Newton-Schulz kernel + error word
+    for (int i = 0; i < 2; ++i) t_kl[i] = sc.take((size_t)d.b * Tcap * d.d * esz);   // k * lr0, k * lr2 of the current update
+    t_ca = muon ? sc.take(sq3 * nsz) : 0;                   // c * A of the current Newton-Schulz iteration
     scratch_bytes = sc.off + 256;
     return 0;
   }
@@ -436,6 +439,7 @@ struct NsIter {
   float ca, cb, cc;
   const float* xf_in; const void* xb_in;           // X: fp32 iterate and its copy in the GEMM type
   void* ab; void* bb;                              // A and B of this iteration (GEMM type)
+  void* cab;                                       // c * A (GEMM type): the left operand of (c * A) @ A, a tensor of its own in the reference
   float* xf_out; void* xb_out; float* u_out;       // X': fp32, GEMM type, and fp32 in the original orientation (each nullable)
 };
 // TN: GEMM operand type of the iteration (bf16 as in the reference, or fp32 for the exact mode)
@@ -446,13 +450,14 @@ void ns_iteration(const NsIter& I, hipStream_t s) {
     auto p = row_params<1>();
     set_term(p.t[0], I.xb_in, I.c, xe, I.xb_in, I.c, xe, I.c);
     p.M = I.r; p.N = I.r; p.out = I.ab; p.ldo = I.r; p.bso = se;
+    p.out2 = I.cab; p.alpha2 = I.cc;
     launch_row_gemm<TN, true, 1, EPI_STORE>("ns_gram", p, I.n, s);
   }
-  {
+  {   // B = b * A + (c * A) @ A, ttt_operation.py:60
     auto p = row_params<1>();
-    set_term(p.t[0], I.ab, I.r, se, I.ab, I.r, se, I.r);
+    set_term(p.t[0], I.cab, I.r, se, I.ab, I.r, se, I.r);
     p.M = I.r; p.N = I.r; p.out = I.bb; p.ldo = I.r; p.bso = se;
-    p.aux = I.ab; p.ldaux = I.r; p.bsaux = se; p.alpha = I.cc; p.beta = I.cb;
+    p.aux = I.ab; p.ldaux = I.r; p.bsaux = se; p.alpha = 1.f; p.beta = I.cb;
     launch_row_gemm<TN, true, 1, EPI_AXPBY>("ns_poly", p, I.n, s);
   }
   {
@@ -602,7 +607,7 @@ struct Runner {
   TN* ab(int u, int it) const { return reinterpret_cast<TN*>(sv + P.s_ab) + ((size_t)u * std::max(1, P.S) + it) * sq3(); }
   TN* bb(int u, int it) const { return reinterpret_cast<TN*>(sv + P.s_bb) + ((size_t)u * std::max(1, P.S) + it) * sq3(); }
   T* h(int i) const { return reinterpret_cast<T*>(sc + hsel[i]); }
-  // kept array i (0..2: lr-scaled operands, 3..5: pre-activations) of update u; batch stride pre_bs(u)
+  // kept array i (0..2: lr-scaled operands, 3..5: pre-activations, 6..7: unscaled operands 0 and 2) of update u; batch stride pre_bs(u)
   T* pre(int u, int i) const { return reinterpret_cast<T*>(sv + P.s_pre[u]) + (size_t)i * d.b * P.pre_T[u] * d.dh; }
   long long pre_bs(int u) const { return (long long)P.pre_T[u] * d.dh; }
   static constexpr bool kBf16 = std::is_same<T, uint16_t>::value;
@@ -867,14 +872,21 @@ struct Runner {
       // ---- update
       const T* kc = k + (size_t)st.start * d.k_ld;
       const T* vc = v + (size_t)st.start * d.v_ld;
+      T* kl0 = scr<T>(P.t_kl[0]);
+      T* kl2 = scr<T>(P.t_kl[1]);
+      const long long klbs = (long long)P.Tcap * d.d;
+      LACT_LAUNCH("k_lr_scale_rows", "update_lr_k", 0.0, (k_lr_scale_rows<T>), dim3((unsigned)(((long long)T_ * d.d / 4 + 255) / 256), d.b), dim3(256), s,
+                  kc, d.k_ld, d.k_bs, lr0 + st.start, lr2 + st.start, (long long)d.kv_len, T_, d.d, kl0, kl2, klbs);
       {
         HiddenParams hp = hidden_params(T_, kc, d.k_ld, d.k_bs, vc, d.v_ld, d.v_bs, ver);
         hp.lr0 = lr0 + st.start; hp.lr1 = lr1 + st.start; hp.lr2 = lr2 + st.start; hp.bslr = d.kv_len;
+        // operands of the three gradient GEMMs: dgate_before_act, hidden * lr1, dhidden_before_mul
         T* z0 = h(0); T* z1 = h(1); T* z2 = h(2);
         long long zbs = hbs();
         if (P.keep_pre) {
-          z0 = pre(u, 0); z1 = pre(u, 1); z2 = pre(u, 2); zbs = pre_bs(u);
+          z0 = pre(u, 6); z1 = pre(u, 1); z2 = pre(u, 7); zbs = pre_bs(u);
           hp.O3 = pre(u, 3); hp.O4 = pre(u, 4); hp.O5 = pre(u, 5);
+          hp.O6 = pre(u, 0); hp.O7 = pre(u, 2);
           hp.bso = zbs;
         }
         hp.O0 = z0; hp.O1 = z1; hp.O2 = z2;
@@ -890,11 +902,11 @@ struct Runner {
         memset(jobs, 0, sizeof(jobs));
         jobs[0].nterms = jobs[1].nterms = jobs[2].nterms = 1;
         jobs[0].M = d.dh; jobs[0].N = d.d;
-        set_tr_term(jobs[0].t[0], upd_z[0], d.dh, upd_zbs, kc, d.k_ld, d.k_bs);
+        set_tr_term(jobs[0].t[0], upd_z[0], d.dh, upd_zbs, kl0, d.d, klbs);
         jobs[1].M = d.d; jobs[1].N = d.dh;
         set_tr_term(jobs[1].t[0], vc, d.v_ld, d.v_bs, upd_z[1], d.dh, upd_zbs);
         jobs[2].M = d.dh; jobs[2].N = d.d;
-        set_tr_term(jobs[2].t[0], upd_z[2], d.dh, upd_zbs, kc, d.k_ld, d.k_bs);
+        set_tr_term(jobs[2].t[0], upd_z[2], d.dh, upd_zbs, kl2, d.d, klbs);
         // square shapes with Muon: the momentum step can ride in the reduction's epilogue (every tile exists for
         // every matrix, and the Newton-Schulz orientation is the packed one)
         PrepFold pf;
@@ -949,6 +961,7 @@ struct Runner {
               f.xf[0] = scr<float>(P.t_xf[0]) + B.xoff; f.xf[1] = scr<float>(P.t_xf[1]) + B.xoff;
               f.xb = xb(u, 0) + B.xoff; f.xb_it_stride = (long long)P.mat3;
               f.ab = ab(u, 0) + B.sqoff; f.bb = bb(u, 0) + B.sqoff; f.sq_it_stride = (long long)sq3();
+              f.cab = scr<uint16_t>(P.t_ca) + B.sqoff;
               f.u_out = usave(u) + B.xoff;
               if (scale_in_kernel) {
                 f.g16 = reinterpret_cast<const uint16_t*>(g16(u)) + B.xoff;
@@ -966,7 +979,7 @@ struct Runner {
             I.n = B.n; I.r = B.r; I.c = B.c; I.nb_for_mask = B.nb; I.mask = B.mask; I.plain = d.ns_mode == LACT_NS_PLAIN_BF16;
             I.ca = P.coeffs[3 * it]; I.cb = P.coeffs[3 * it + 1]; I.cc = P.coeffs[3 * it + 2];
             I.xf_in = scr<float>(P.t_xf[it & 1]) + B.xoff; I.xb_in = xb(u, it) + B.xoff;
-            I.ab = ab(u, it) + B.sqoff; I.bb = bb(u, it) + B.sqoff;
+            I.ab = ab(u, it) + B.sqoff; I.bb = bb(u, it) + B.sqoff; I.cab = scr<TN>(P.t_ca) + B.sqoff;
             I.xf_out = last ? nullptr : scr<float>(P.t_xf[(it + 1) & 1]) + B.xoff;
             I.xb_out = last ? (void*)(scr<TN>(P.t_xbtmp) + B.xoff) : (void*)(xb(u, it + 1) + B.xoff);
             I.u_out = last ? usave(u) + B.xoff : nullptr;
@@ -1547,7 +1560,7 @@ namespace {
 struct NsPlan {
   MatGeom g;
   int r, c, nblk;
-  size_t o_g16, o_ss, o_norm, o_xf[2], o_xb[2], o_ab, o_bb, bytes;
+  size_t o_g16, o_ss, o_norm, o_xf[2], o_xb[2], o_ab, o_bb, o_ca, bytes;
   void build(int n, int rows, int cols) {
     // one "matrix kind" (index 0) of shape [rows, cols]: d = cols, dh = rows
     g.d = cols; g.dh = rows; g.nb = n; g.elems = (long long)rows * cols; g.stacked = 0;
@@ -1557,7 +1570,7 @@ struct NsPlan {
     const size_t e = (size_t)n * g.elems;
     o_g16 = b.take(e * 4); o_ss = b.take((size_t)n * nblk * 4); o_norm = b.take((size_t)n * 4);
     o_xf[0] = b.take(e * 4); o_xf[1] = b.take(e * 4); o_xb[0] = b.take(e * 4); o_xb[1] = b.take(e * 4);
-    o_ab = b.take((size_t)n * r * r * 4); o_bb = b.take((size_t)n * r * r * 4);
+    o_ab = b.take((size_t)n * r * r * 4); o_bb = b.take((size_t)n * r * r * 4); o_ca = b.take((size_t)n * r * r * 4);
     bytes = b.off + 256;
   }
 };
@@ -1591,7 +1604,7 @@ int newton_schulz_t(int32_t n, int32_t rows, int32_t cols, const float* gin, flo
     I.ca = coeffs[3 * it]; I.cb = coeffs[3 * it + 1]; I.cc = coeffs[3 * it + 2];
     I.xf_in = reinterpret_cast<float*>(ws + P.o_xf[it & 1]);
     I.xb_in = ws + P.o_xb[it & 1];
-    I.ab = ws + P.o_ab; I.bb = ws + P.o_bb;
+    I.ab = ws + P.o_ab; I.bb = ws + P.o_bb; I.cab = ws + P.o_ca;
     I.xf_out = last ? nullptr : reinterpret_cast<float*>(ws + P.o_xf[(it + 1) & 1]);
     I.xb_out = last ? nullptr : ws + P.o_xb[(it + 1) & 1];
     I.u_out = last ? out : nullptr;

@@ -43,6 +43,7 @@ struct NsFusedParams {
   float* xf[2];
   uint16_t* xb; long long xb_it_stride;            // X_k at xb + k * xb_it_stride, k < S
   uint16_t* ab; uint16_t* bb; long long sq_it_stride;
+  uint16_t* cab;                                   // forward: c * A of the running iteration (one [r, r] buffer per matrix)
   float* u_out;                                    // X_S, fp32, original orientation
   // backward: incoming gradient in gxf[0] / gxb[0]; the result ends in gxf[S & 1]
   float* gxf[2]; uint16_t* gxb[2]; uint16_t* sg; uint16_t* gas;
@@ -108,6 +109,7 @@ __device__ __forceinline__ RowGemmDmaParams<NT> ns_row_params() {
   RowGemmDmaParams<NT> q;
   q.g.accumulate = 0; q.g.aux = nullptr; q.g.ldaux = 0; q.g.bsaux = 0; q.g.alpha = 1.f; q.g.beta = 0.f;
   q.g.out_c = nullptr; q.g.out_t = nullptr; q.g.transpose_mask = 0; q.g.nb = 1; q.g.round_out_bf16 = 0;
+  q.g.out2 = nullptr; q.g.alpha2 = 0.f;
   q.out_ct = nullptr;
   return q;
 }
@@ -145,7 +147,6 @@ __global__ __launch_bounds__(DMA_THREADS) void k_ns_fused(const NsFusedParams p)
     if (member == 0 && threadIdx.x == 0) p.norms[z] = n;
     float den = n + 1e-7f;
     if (p.plain) den = round_bf16(den);
-    const float inv = 1.f / den;
     const size_t zo = (size_t)z * p.r * p.c + (size_t)rx * TS::BM * p.c + ry * TS::BN;
     constexpr int GR = TS::BN / 8;   // 16-byte granules per tile row
     for (int id = threadIdx.x; id < TS::BM * GR; id += DMA_THREADS) {
@@ -155,8 +156,8 @@ __global__ __launch_bounds__(DMA_THREADS) void k_ns_fused(const NsFusedParams p)
       float v[8];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        v[2 * i] = __uint_as_float(w[i] << 16) * inv;
-        v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u) * inv;
+        v[2 * i] = __fdiv_rn(__uint_as_float(w[i] << 16), den);            // the quotient itself (ttt_operation.py:49), not a product with 1 / den
+        v[2 * i + 1] = __fdiv_rn(__uint_as_float(w[i] & 0xffff0000u), den);
       }
       if (p.plain) {
 #pragma unroll
@@ -187,6 +188,7 @@ __global__ __launch_bounds__(DMA_THREADS) void k_ns_fused(const NsFusedParams p)
         auto q = ns_row_params<1>();
         ns_term(q.g.t[0], X, c, xe, X, c, xe, c);
         q.g.M = r; q.g.N = r; q.g.out = A; q.g.ldo = r; q.g.bso = se;
+        q.g.out2 = p.cab; q.g.alpha2 = cc;
         row_gemm_tile<TS, 1, EPI_STORE, false, true>(q, sx, sy, z, smem);
       }
       LACT_NS_TS(1 + step * 6 + 0);
@@ -194,9 +196,9 @@ __global__ __launch_bounds__(DMA_THREADS) void k_ns_fused(const NsFusedParams p)
       LACT_NS_TS(1 + step * 6 + 1);
       if (sq_tile) {
         auto q = ns_row_params<1>();
-        ns_term(q.g.t[0], A, r, se, A, r, se, r);
+        ns_term(q.g.t[0], p.cab, r, se, A, r, se, r);
         q.g.M = r; q.g.N = r; q.g.out = B; q.g.ldo = r; q.g.bso = se;
-        q.g.aux = A; q.g.ldaux = r; q.g.bsaux = se; q.g.alpha = cc; q.g.beta = cb;
+        q.g.aux = A; q.g.ldaux = r; q.g.bsaux = se; q.g.alpha = 1.f; q.g.beta = cb;
         row_gemm_tile<TS, 1, EPI_AXPBY, false, true>(q, sx, sy, z, smem);
       }
       LACT_NS_TS(1 + step * 6 + 2);
@@ -299,10 +301,11 @@ __global__ __launch_bounds__(DMA_THREADS) void k_ns_fused(const NsFusedParams p)
         if (id < TS::BM * GR) {
           const size_t o = zo + (size_t)(id / GR) * p.c + (id % GR) * 8;
           const uint32_t w[4] = {gi[t].x, gi[t].y, gi[t].z, gi[t].w};
-          float4 v0 = make_float4(ga[t].x * c0 - __uint_as_float(w[0] << 16) * c1, ga[t].y * c0 - __uint_as_float(w[0] & 0xffff0000u) * c1,
-                                  ga[t].z * c0 - __uint_as_float(w[1] << 16) * c1, ga[t].w * c0 - __uint_as_float(w[1] & 0xffff0000u) * c1);
-          float4 v1 = make_float4(gb[t].x * c0 - __uint_as_float(w[2] << 16) * c1, gb[t].y * c0 - __uint_as_float(w[2] & 0xffff0000u) * c1,
-                                  gb[t].z * c0 - __uint_as_float(w[3] << 16) * c1, gb[t].w * c0 - __uint_as_float(w[3] & 0xffff0000u) * c1);
+          // the gradient that leaves Newton-Schulz through its input cast (G.bfloat16()) has that type
+          float4 v0 = make_float4(round_bf16(ga[t].x * c0 - __uint_as_float(w[0] << 16) * c1), round_bf16(ga[t].y * c0 - __uint_as_float(w[0] & 0xffff0000u) * c1),
+                                  round_bf16(ga[t].z * c0 - __uint_as_float(w[1] << 16) * c1), round_bf16(ga[t].w * c0 - __uint_as_float(w[1] & 0xffff0000u) * c1));
+          float4 v1 = make_float4(round_bf16(gb[t].x * c0 - __uint_as_float(w[2] << 16) * c1), round_bf16(gb[t].y * c0 - __uint_as_float(w[2] & 0xffff0000u) * c1),
+                                  round_bf16(gb[t].z * c0 - __uint_as_float(w[3] << 16) * c1), round_bf16(gb[t].w * c0 - __uint_as_float(w[3] & 0xffff0000u) * c1));
           if (p.gm_carry) {
             if (p.carry_valid) {
               const float4 a = *reinterpret_cast<const float4*>(p.gm_carry + o), b = *reinterpret_cast<const float4*>(p.gm_carry + o + 4);

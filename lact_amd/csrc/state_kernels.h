@@ -144,7 +144,9 @@ __global__ void k_momentum_prep(const MomentumPrepParams p) {
     if (p.round_partial_bf16) v = f4(round_bf16(v.x), round_bf16(v.y), round_bf16(v.z), round_bf16(v.w));
     if (p.m_prev) {
       const float4 m = ld4(p.m_prev + zo + e);
-      v.x += m.x * mb; v.y += m.y * mb; v.z += m.z * mb; v.w += m.w * mb;
+      // product and sum rounded separately, as the reference's two tensor operations are (ttt_operation.py:174-176)
+      v.x = __fadd_rn(v.x, __fmul_rn(m.x, mb)); v.y = __fadd_rn(v.y, __fmul_rn(m.y, mb));
+      v.z = __fadd_rn(v.z, __fmul_rn(m.z, mb)); v.w = __fadd_rn(v.w, __fmul_rn(m.w, mb));
     }
     if (p.d_out) st4(p.d_out + zo + e, v);
     if (ext) st4(ext + e, v);
@@ -190,7 +192,6 @@ __global__ void k_ns_scale(const NsScaleParams p) {
   if (blockIdx.x == 0 && threadIdx.x == 0) p.norms[m] = n;
   float den = n + 1e-7f;
   if (p.plain_bf16) den = round_bf16(den);
-  const float inv = 1.f / den;
   const FlatRange R(p.g.ns_elems(m));
   const size_t zo = p.g.ns_base(m);
   // `u` (only when zero iterations follow; never stacked): original orientation of matrix m = packed z
@@ -201,7 +202,7 @@ __global__ void k_ns_scale(const NsScaleParams p) {
     Elem<TN>::load4(reinterpret_cast<const TN*>(p.g16) + zo + x, v);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      v[i] *= inv;
+      v[i] = __fdiv_rn(v[i], den);   // the quotient itself (ttt_operation.py:49), not a product with 1 / den
       if (p.plain_bf16) v[i] = round_bf16(v[i]);
     }
     st4(p.xf + zo + x, f4(v[0], v[1], v[2], v[3]));
@@ -474,7 +475,9 @@ __global__ void k_grad_prep(const GradPrepParams p) {
         }
         gx = f4(t[0], t[1], t[2], t[3]);
       }
-      gv = f4(gx.x * c0 - g[0] * c1, gx.y * c0 - g[1] * c1, gx.z * c0 - g[2] * c1, gx.w * c0 - g[3] * c1);
+      // the gradient that leaves Newton-Schulz through its input cast (G.bfloat16(), ttt_operation.py:45) has that type
+      gv = f4(Elem<TN>::rnd(gx.x * c0 - g[0] * c1), Elem<TN>::rnd(gx.y * c0 - g[1] * c1), Elem<TN>::rnd(gx.z * c0 - g[2] * c1),
+              Elem<TN>::rnd(gx.w * c0 - g[3] * c1));
       if (p.cr != 0.f) {
         const float4 w = ld4(p.gw_hat + o);
         gv.x += p.cr * w.x; gv.y += p.cr * w.y; gv.z += p.cr * w.z; gv.w += p.cr * w.w;

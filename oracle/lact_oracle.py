@@ -67,20 +67,74 @@ TTTOperator = collections.namedtuple("TTTOperator", ["start", "end", "update", "
 class Numerics:
     autocast: bool = False
     ns_dtype: Optional[torch.dtype] = torch.bfloat16
+    # How a bf16 GEMM accumulates.  Every choice rounds at the same points (bf16 operands, bf16 result); only the
+    # order / width of the additions in between differs, as it does between any two GEMM libraries:
+    #   "fp32"    one fp32 matmul (the CPU library's own blocking)
+    #   "fp64"    float64 accumulation
+    #   "kblockN"  fp32 partial products over N consecutive k, added in ascending order (N = 16: what a
+    #             matrix-core instruction with K = 16 does)
+    #   "kblockNr" the same, added in descending order
+    # tests/ use the spread between these ("order-only floor") as the yardstick for the Muon path, where
+    # Newton-Schulz amplifies single bf16 rounding flips to percent level.
+    accumulate: str = "fp32"
+
+    def _ordered_mm(self, a: torch.Tensor, b: torch.Tensor, out_dtype) -> torch.Tensor:
+        """a @ b on fp32 values with the accumulation order named by `accumulate`, result cast to out_dtype."""
+        if self.accumulate == "fp32":
+            return torch.matmul(a.float(), b.float()).to(out_dtype)
+        if self.accumulate == "fp64":
+            return torch.matmul(a.double(), b.double()).to(out_dtype)
+        blk = int(self.accumulate[len("kblock"):].rstrip("r"))
+        af, bfl = a.float(), b.float()
+        starts = list(range(0, af.shape[-1], blk))
+        if self.accumulate.endswith("r"):
+            starts.reverse()
+        acc = None
+        for s0 in starts:
+            part = torch.matmul(af[..., s0:s0 + blk], bfl[..., s0:s0 + blk, :])
+            acc = part if acc is None else acc + part
+        return acc.to(out_dtype)
 
     def mm(self, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
         """Batched matmul with the autocast policy of `aten::bmm` (lower-precision list)."""
         if self.autocast:
             # bf16-rounded operands, fp32 accumulation, bf16 result (what a GPU bf16 GEMM does);
             # done as an fp32 GEMM on rounded values so that the CPU run is fast and deterministic.
-            return torch.matmul(a.bfloat16().float(), b.bfloat16().float()).bfloat16()
+            return self._ordered_mm(a.bfloat16(), b.bfloat16(), torch.bfloat16)
+        if self.accumulate != "fp32" and a.dtype == b.dtype and a.dtype in (torch.bfloat16, torch.float32):
+            return self._ordered_mm(a, b, a.dtype)     # no autocast: a bf16 (Newton-Schulz) or fp32 GEMM, reordered
         return torch.matmul(a, b)
 
     def norm(self, x: torch.Tensor, dim, keepdim=True) -> torch.Tensor:
-        """Autocast keeps norms in fp32 (ttt_operation.py:26 "norm will upcast to float32")."""
-        if self.autocast:
-            return x.float().norm(dim=dim, keepdim=keepdim)
-        return x.norm(dim=dim, keepdim=keepdim)
+        """Autocast keeps norms in fp32 (ttt_operation.py:26 "norm will upcast to float32").  The accumulation
+        variants change the order / width of the sum of squares too (the result moves by an ulp or so)."""
+        xf = x.float() if self.autocast else x
+        if self.accumulate == "fp32" or xf.dtype == torch.float64:
+            return xf.norm(dim=dim, keepdim=keepdim)
+        out_dtype = xf.dtype
+        dims = (dim,) if isinstance(dim, int) else tuple(dim)
+        sq = xf.double() ** 2
+        if self.accumulate == "fp64":
+            ss = sq.sum(dim=dims, keepdim=keepdim)
+            return ss.sqrt().float().to(out_dtype)
+        # fp32 partial sums over blocks of consecutive elements, added in ascending / descending order
+        blk = int(self.accumulate[len("kblock"):].rstrip("r")) * 8
+        dims = tuple(d % x.dim() for d in dims)
+        keep = [d for d in range(x.dim()) if d not in dims]
+        flat = xf.float().permute(*keep, *dims).reshape(*[x.shape[d] for d in keep], -1)
+        flat = flat * flat
+        starts = list(range(0, flat.shape[-1], blk))
+        if self.accumulate.endswith("r"):
+            starts.reverse()
+        acc = None
+        for s0 in starts:
+            part = flat[..., s0:s0 + blk].sum(dim=-1)
+            acc = part if acc is None else acc + part
+        n = acc.sqrt()
+        if keepdim:
+            for d in sorted(dims):
+                n = n.unsqueeze(d)
+        return n.to(out_dtype)
 
 
 # ---------------------------------------------------------------------------------------------
@@ -479,6 +533,14 @@ def make_inputs(b: int, L: int, d: int, dh: int, *, seed: int, act_dtype=torch.b
     mom = None if momentum_value is None else torch.full((b, L, 1), float(momentum_value))
     return dict(w0=w0, w1=w1, w2=w2, q=q.to(act_dtype), k=k.to(act_dtype), v=v.to(act_dtype),
                 lr0=lr0, lr1=lr1, lr2=lr2, momentum=mom)
+
+
+ORDER_VARIANTS = ("fp64", "kblock16", "kblock64r")
+
+
+def order_variants(num: Numerics):
+    """The same numerics with each of the other accumulation orders (see Numerics.accumulate)."""
+    return [Numerics(autocast=num.autocast, ns_dtype=num.ns_dtype, accumulate=a) for a in ORDER_VARIANTS]
 
 
 def rel_l2(a: torch.Tensor, ref: torch.Tensor) -> float:

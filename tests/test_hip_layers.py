@@ -170,9 +170,31 @@ def test_bidirectional_layer_against_reference_golden(tag):
     res = grads_and_out(layer, x.to(DEV), go.to(DEV))
     errs = compare(res, ref)
     say("  ", errs)
-    # Muon: bf16 Newton-Schulz on both sides, 16 x 24 matrices: two roundings of the same iteration differ by several
-    # percent there (the exact-arithmetic Muon check is test_*_layer_against_oracle below)
-    assert max(errs.values()) < (0.15 if kw["use_muon"] else 2e-4)
+    if not kw["use_muon"]:
+        assert max(errs.values()) < 2e-4
+        return
+    # Muon: bf16 Newton-Schulz on both sides, here on 16 x 24 matrices whose forward comes out without a single
+    # rounding flip: the output meets the fp32 bound outright.
+    assert errs["y"] < 2e-4
+    # The gradients pass through the backward of the bf16 iteration.  The HIP backward is a closed form that rounds
+    # each of its three products per iteration once; autograd rounds every partial product and every gradient
+    # accumulation of the same iteration (about as many roundings, at other points), so the two are independent
+    # realisations of the same bf16 noise, each as far from float64 arithmetic as the other.  Yardstick: the larger of
+    # the order-only floor (oracle against itself, accumulation order changed, O.order_variants) and the oracle's own
+    # distance from the float64 oracle, per entry.
+    def oracle_run(num, dt=torch.float32):
+        ol = LO.BidirectionalLaCTSwiGLU(num=num, **kw).to(dt)
+        ol.load_state_dict({k_: v_.to(dt) for k_, v_ in params.items()}, strict=True)
+        return grads_and_out(ol, x.to(dt), go.to(dt))
+    base = oracle_run(PLAIN)
+    f64 = oracle_run(EXACT, torch.float64)
+    yard = compare(base, f64)
+    for v in O.order_variants(PLAIN):
+        for n, e in compare(oracle_run(v), base).items():
+            yard[n] = max(yard[n], e)
+    say("   yardstick", yard, "oracle vs reference", compare(base, ref), "hip vs f64", compare(res, f64))
+    for n, e in errs.items():
+        assert e <= 1.5 * yard[n] + 1e-3, (n, e, yard[n])
 
 
 @pytest.mark.parametrize("use_muon,use_o_norm,qk_l2", [(False, True, True), (False, False, False), (True, True, True)])

@@ -384,3 +384,34 @@ def test_carried_momentum_state_composes_and_is_the_heavy_ball_step():
     assert all(float(zeros[4 + j].abs().max()) == 0.0 for j in range(3))
     off = fn(w0, w1, w2, q, k, v, lr0, lr1, lr2, 0.7, 1, 24, True, False, 3, True, None, None, None, None, False, **kw)
     assert off[4] is None and off[5] is None and off[6] is None
+
+
+# ---- the order-only floor of the bf16 Muon path -------------------------------------------------------------
+@pytest.mark.parametrize("b,L,d,dh,C", [(2, 3 * 64 + 5, 64, 64, 64), (2, 1024, 384, 384, 512)])
+def test_order_only_floor_of_bf16_newton_schulz(b, L, d, dh, C):
+    """How far the oracle moves when NOTHING changes but the order in which its bf16 GEMMs and its norms add their
+    terms (same operands, same rounding points): float64 accumulation, K blocks of 16 ascending, K blocks of 64
+    descending.  Without Muon that is the fp32 summation noise (below 1e-3 on every output); with Muon the
+    Newton-Schulz iteration magnifies single bf16 rounding flips to about 1e-2 on the output -- the size of the
+    north-star bf16 tolerance itself.  The GPU parity tests state their Muon bound as 1.5 x this floor, measured on
+    their own inputs; here its size is pinned so that it cannot be inflated unnoticed (an order variant that also
+    moved a rounding point would show up in the Muon-off leg, which must stay at summation-noise level)."""
+    inp = O.make_inputs(b, L, d, dh, seed=7, act_dtype=torch.bfloat16, momentum_value=None)
+    inp["momentum"] = torch.sigmoid(torch.randn(b, L, 1, generator=torch.Generator().manual_seed(106)) + 1.5)
+    order = ("w0", "w1", "w2", "q", "k", "v", "lr0", "lr1", "lr2")
+    steps = O.block_causal_steps(L, C)
+    base = O.Numerics(autocast=True)
+    for muon in (False, True):
+        run = lambda num: O.run_program(*[inp[n] for n in order], steps, num=num, momentum=inp["momentum"],
+                                        ns_coeffs=O.NS5_COEFFS if muon else None)
+        ref_out, ref_w, _ = run(base)
+        f_out, f_w = 0.0, 0.0
+        for v in O.order_variants(base):
+            out, ws, _ = run(v)
+            f_out = max(f_out, O.rel_l2(out, ref_out))
+            f_w = max(f_w, max(O.rel_l2(a, r) for a, r in zip(ws, ref_w)))
+        print(f"order-only floor d={d} muon={muon}: output {f_out:.2e}, fast weights {f_w:.2e}")
+        if muon:
+            assert 3e-3 < f_out < 4e-2 and 3e-3 < f_w < 4e-2
+        else:
+            assert f_out < 1e-3 and f_w < 1e-4
