@@ -121,6 +121,18 @@ size_t lact_newton_schulz_workspace_bytes(int32_t n, int32_t rows, int32_t cols,
 int lact_newton_schulz(int32_t n, int32_t rows, int32_t cols, const float* g, float* out, int32_t steps,
                        const float* coeffs, int32_t ns_mode, void* workspace, void* stream);
 
+/* lact_newton_schulz for callers that cannot allocate device memory or hand over a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The workspace is
+ * a fixed array of LACT_NS_STATIC_WORKSPACE_BYTES in device memory that the library holds on every GPU it runs on
+ * until the process ends; the call allocates nothing.  Shapes whose lact_newton_schulz_workspace_bytes exceed it are
+ * refused (return value < 0, message in lact_last_error).  Every call on a GPU uses that GPU's one array: calls that
+ * overlap on one GPU (two streams, two threads) race; calls on one stream are ordered by the stream.  Same kernels
+ * and same results, bit for bit, as lact_newton_schulz. */
+#define LACT_NS_STATIC_WORKSPACE_BYTES (32u << 20)
+size_t lact_newton_schulz_static_capacity(void);
+int lact_newton_schulz_static(int32_t n, int32_t rows, int32_t cols, const float* g, float* out, int32_t steps,
+                              const float* coeffs, int32_t ns_mode, void* stream);
+
 /* ---- Layer pre- and post-processing (the tensor code of the layer classes around the operation, one pass each;
  * in the reference a chain of PyTorch ops in the layers' forward, with autograd for the backward).
  * act_dtype as above; head dim a multiple of 4, at most 1024.  All buffers contiguous.

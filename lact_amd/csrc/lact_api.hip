@@ -1616,6 +1616,36 @@ int newton_schulz_t(int32_t n, int32_t rows, int32_t cols, const float* gin, flo
 }  // namespace
 
 
+// ---- Newton-Schulz without a caller workspace: the workspace is a fixed array in device memory -------------
+// Every GPU the library runs on holds its own copy of the array (at its own address) until the process ends.
+// In host code the array's name is only a handle for hipGetSymbolAddress; the address it returns for the current
+// device is what kernels and copies get.
+static __device__ __align__(256) unsigned char scratch[LACT_NS_STATIC_WORKSPACE_BYTES];
+namespace {
+std::mutex g_static_ws_mutex;
+void* g_static_ws[64] = {};   // per device: address of `scratch` there
+// Address of the static workspace on the current device (looked up once per device), or null with the error set.
+void* static_workspace() {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= 64) {
+    fail("static workspace: no current device (or device index beyond 63)");
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_static_ws_mutex);
+  if (!g_static_ws[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      fail(std::string("static workspace: hipGetSymbolAddress failed: ") + hipGetErrorString(e));
+      return nullptr;
+    }
+    g_static_ws[dev] = ptr;
+  }
+  return g_static_ws[dev];
+}
+}  // namespace
+
 extern "C" {
 
 const char* lact_last_error(void) { return g_err.c_str(); }
@@ -1879,6 +1909,20 @@ int lact_newton_schulz(int32_t n, int32_t rows, int32_t cols, const float* gin, 
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (ns_mode == LACT_NS_FP32) return newton_schulz_t<float>(n, rows, cols, gin, out, steps, coeffs, ns_mode, workspace, s);
   return newton_schulz_t<uint16_t>(n, rows, cols, gin, out, steps, coeffs, ns_mode, workspace, s);
+}
+
+size_t lact_newton_schulz_static_capacity(void) { return LACT_NS_STATIC_WORKSPACE_BYTES; }
+
+int lact_newton_schulz_static(int32_t n, int32_t rows, int32_t cols, const float* gin, float* out, int32_t steps,
+                              const float* coeffs, int32_t ns_mode, void* stream) {
+  const size_t need = lact_newton_schulz_workspace_bytes(n, rows, cols, steps);
+  if (need == 0) return fail("bad Newton-Schulz shape");
+  if (need > LACT_NS_STATIC_WORKSPACE_BYTES)
+    return fail("lact_newton_schulz_static: n x rows x cols needs " + std::to_string(need) + " workspace bytes, the static workspace holds " +
+                std::to_string((size_t)LACT_NS_STATIC_WORKSPACE_BYTES) + " (use lact_newton_schulz with a caller workspace)");
+  void* ws = static_workspace();
+  if (!ws) return -1;
+  return lact_newton_schulz(n, rows, cols, gin, out, steps, coeffs, ns_mode, ws, stream);
 }
 
 }  // extern "C"
