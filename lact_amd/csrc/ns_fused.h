@@ -23,6 +23,7 @@
 // other with an event, so two such kernels never hold compute units while waiting for each other.
 #pragma once
 #include "gemm_dma_kernels.h"
+#include "state_kernels.h"
 
 // Optional in-kernel timestamps (defined only by timing experiments; expands to nothing in the library).
 #ifndef LACT_NS_TS
@@ -302,10 +303,13 @@ __global__ __launch_bounds__(DMA_THREADS) void k_ns_fused(const NsFusedParams p)
           const size_t o = zo + (size_t)(id / GR) * p.c + (id % GR) * 8;
           const uint32_t w[4] = {gi[t].x, gi[t].y, gi[t].z, gi[t].w};
           // the gradient that leaves Newton-Schulz through its input cast (G.bfloat16()) has that type
-          float4 v0 = make_float4(round_bf16(ga[t].x * c0 - __uint_as_float(w[0] << 16) * c1), round_bf16(ga[t].y * c0 - __uint_as_float(w[0] & 0xffff0000u) * c1),
-                                  round_bf16(ga[t].z * c0 - __uint_as_float(w[1] << 16) * c1), round_bf16(ga[t].w * c0 - __uint_as_float(w[1] & 0xffff0000u) * c1));
-          float4 v1 = make_float4(round_bf16(gb[t].x * c0 - __uint_as_float(w[2] << 16) * c1), round_bf16(gb[t].y * c0 - __uint_as_float(w[2] & 0xffff0000u) * c1),
-                                  round_bf16(gb[t].z * c0 - __uint_as_float(w[3] << 16) * c1), round_bf16(gb[t].w * c0 - __uint_as_float(w[3] & 0xffff0000u) * c1));
+          const float gi0 = __uint_as_float(w[0] << 16), gi1 = __uint_as_float(w[0] & 0xffff0000u), gi2 = __uint_as_float(w[1] << 16),
+                      gi3 = __uint_as_float(w[1] & 0xffff0000u), gi4 = __uint_as_float(w[2] << 16), gi5 = __uint_as_float(w[2] & 0xffff0000u),
+                      gi6 = __uint_as_float(w[3] << 16), gi7 = __uint_as_float(w[3] & 0xffff0000u);
+          float4 v0 = make_float4(ns_input_grad<uint16_t>(ga[t].x, gi0, c0, c1), ns_input_grad<uint16_t>(ga[t].y, gi1, c0, c1),
+                                  ns_input_grad<uint16_t>(ga[t].z, gi2, c0, c1), ns_input_grad<uint16_t>(ga[t].w, gi3, c0, c1));
+          float4 v1 = make_float4(ns_input_grad<uint16_t>(gb[t].x, gi4, c0, c1), ns_input_grad<uint16_t>(gb[t].y, gi5, c0, c1),
+                                  ns_input_grad<uint16_t>(gb[t].z, gi6, c0, c1), ns_input_grad<uint16_t>(gb[t].w, gi7, c0, c1));
           if (p.gm_carry) {
             if (p.carry_valid) {
               const float4 a = *reinterpret_cast<const float4*>(p.gm_carry + o), b = *reinterpret_cast<const float4*>(p.gm_carry + o + 4);

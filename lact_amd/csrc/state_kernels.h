@@ -423,6 +423,13 @@ __global__ void k_ns_bwd_dot(const NsDotParams p) {
   if (threadIdx.x == 0) p.dot_part[(size_t)m * gridDim.x + blockIdx.x] = s;
 }
 
+// Gradient w.r.t. the Newton-Schulz input G16 (type TN) of X0 = G16 / (|G16| + 1e-7), from the gradient gx of X0:
+// gx * c0 through the quotient, -g16 * c1 through the norm (c0 = 1 / (n + eps), c1 = <gx, G16> / (n (n + eps)^2)).
+template <typename TN>
+__device__ __forceinline__ float ns_input_grad(float gx, float g16, float c0, float c1) {
+  return Elem<TN>::rnd(Elem<TN>::rnd(gx * c0) - Elem<TN>::rnd(g16 * c1));
+}
+
 struct GradPrepParams {
   MatGeom g;
   int muon;
@@ -476,8 +483,9 @@ __global__ void k_grad_prep(const GradPrepParams p) {
         gx = f4(t[0], t[1], t[2], t[3]);
       }
       // the gradient that leaves Newton-Schulz through its input cast (G.bfloat16(), ttt_operation.py:45) has that type
-      gv = f4(Elem<TN>::rnd(gx.x * c0 - g[0] * c1), Elem<TN>::rnd(gx.y * c0 - g[1] * c1), Elem<TN>::rnd(gx.z * c0 - g[2] * c1),
-              Elem<TN>::rnd(gx.w * c0 - g[3] * c1));
+      // (two gradients arrive there, through the quotient and through the norm, :49; each is a tensor of that type, and so is their sum)
+      gv = f4(ns_input_grad<TN>(gx.x, g[0], c0, c1), ns_input_grad<TN>(gx.y, g[1], c0, c1), ns_input_grad<TN>(gx.z, g[2], c0, c1),
+              ns_input_grad<TN>(gx.w, g[3], c0, c1));
       if (p.cr != 0.f) {
         const float4 w = ld4(p.gw_hat + o);
         gv.x += p.cr * w.x; gv.y += p.cr * w.y; gv.z += p.cr * w.z; gv.w += p.cr * w.w;

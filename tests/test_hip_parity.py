@@ -326,6 +326,64 @@ def test_bidirectional_golden_vectors(tag):
     assert e <= 1.5 * floor + 1e-3
 
 
+# ---- golden vectors of the LLM operations and the NVS program, written from the reference (CPU, fp32) ------------
+from test_oracle_pins import LLM_TAGS, NVS_TAGS, load_llm_nvs_gold, run_oracle_on_gold  # noqa: E402
+
+
+@pytest.mark.parametrize("tag", LLM_TAGS + NVS_TAGS)
+def test_llm_and_nvs_golden_vectors(tag):
+    """tests/golden/make_llm_nvs_golden.py: the reference's own block_causal_lact_swiglu /
+    prenorm_block_causal_lact_swiglu (ttt_operation.py:71-364) and NVS program (lact_ttt.py:71-147) on the CPU in
+    fp32: outputs, returned weights and the gradient of every input.  Without Newton-Schulz the fp32 bound holds;
+    with it (bf16 on both sides) the order-only floor around the reference's vectors is the yardstick."""
+    say("llm / nvs golden", tag)
+    t, outs, gos, grads, meta = load_llm_nvs_gold(tag)
+    g = {n: v.to(DEV).requires_grad_(True) for n, v in t.items()}
+    if tag.startswith("llm"):
+        fn = T.prenorm_block_causal_lact_swiglu if bool(meta["prenorm"]) else T.block_causal_lact_swiglu
+        res = [fn(*args9(g), int(meta["chunk"]), bool(meta["use_muon"]), g.get("momentum"))]
+        bf16_ns = bool(meta["use_muon"])
+    else:
+        order = [nvs.TTTOperator(int(s0), int(e0), bool(u), bool(ap)) for s0, e0, u, ap in meta["order"]]
+        res = list(nvs.fast_weight_swish_glu_weight_norm_mini_batch_apply(*args9(g), order, int(meta["steps"])))
+        bf16_ns = True           # lact_ttt.py:117-126 casts to bf16 and normalises even with zero iterations
+    loss = sum((r.float() * go.to(DEV)).sum() for r, go in zip(res, gos))
+    names = list(grads)
+    got = dict(zip(names, torch.autograd.grad(loss, [g[n] for n in names])))
+    errs = {f"out{i}": O.rel_l2(r, o) for i, (r, o) in enumerate(zip(res, outs))}
+    errs.update({n: O.rel_l2(got[n], grads[n]) for n in names if float(grads[n].norm()) > 0})
+    say("  ", {n: float("%.2e" % e) for n, e in errs.items()})
+    if not bf16_ns:
+        assert max(errs.values()) < 1e-4
+        return
+    yard = {n: 0.0 for n in errs}
+    for v in O.order_variants(PLAIN):
+        tt, r = run_oracle_on_gold(tag, t, meta, num=v)
+        l = sum((x.float() * go).sum() for x, go in zip(r, gos))
+        gv = dict(zip(names, torch.autograd.grad(l, [tt[n] for n in names])))
+        for i, (x, o) in enumerate(zip(r, outs)):
+            yard[f"out{i}"] = max(yard[f"out{i}"], O.rel_l2(x, o))
+        for n in names:
+            if n in yard:
+                yard[n] = max(yard[n], O.rel_l2(gv[n], grads[n]))
+    say("   order-only floor", {n: float("%.2e" % e) for n, e in yard.items()})
+    # Gradients pass through the backward of the bf16 iteration, where the closed-form HIP backward rounds each of its
+    # three products per iteration once and autograd rounds every partial product and every gradient accumulation:
+    # as many roundings at other points, i.e. another realisation of the same noise.  On matrices this small the
+    # forward comes out without a single flip (outputs and weights above agree to fp32 round-off) and the order-only
+    # floor is far below that noise, so for the gradients the yardstick is the larger of the floor and the distance
+    # of the reference's own vectors from float64 arithmetic.
+    t64, r64 = run_oracle_on_gold(tag, {n: v.double() for n, v in t.items()}, meta, num=EXACT)
+    l64 = sum((x * go.double()).sum() for x, go in zip(r64, gos))
+    g64 = dict(zip(names, torch.autograd.grad(l64, [t64[n] for n in names])))
+    for n in names:
+        if n in yard:
+            yard[n] = max(yard[n], O.rel_l2(grads[n], g64[n]))
+    say("   gradient yardstick", {n: float("%.2e" % yard[n]) for n in names if n in yard})
+    for n, e in errs.items():
+        assert e <= (2.0 if n == "momentum" else 1.5) * yard[n] + 1e-3, (n, e, yard[n])
+
+
 # ---- NVS program (config 3 shape family) -----------------------------------------------------------
 def test_nvs_program_returns_weights_and_grads():
     say("nvs program")
@@ -783,6 +841,22 @@ def full_size_properties(b, L, d, dh, C, seed, single_update):
     else:
         # the first chunk's momentum weighs no earlier state; later chunks' momentum does
         assert float(gr1["momentum"][:, :C].abs().max()) == 0.0 and float(gr1["momentum"][:, C:last].abs().max()) > 0.0
+
+
+@pytest.mark.parametrize("cfg,b,L,d,dh,C,seed", [
+    (1, 16, 4096, 384, 384, 2048, 1001),          # config 1 whole: one update, two applies
+    (2, 4, 3 * 2048, 384, 384, 2048, 1002),       # config 2, first three chunks: two chained updates with momentum carry
+    (4, 12, 3 * 4680, 128, 256, 4680, 1004)])     # config 4, first three chunks (73 x 64 + 8 tokens each)
+def test_config_full_size_against_oracle(cfg, b, L, d, dh, C, seed):
+    """The benchmark shapes at their full b, d, dh and chunk size (Muon, momentum 0.9, bf16, forward + backward):
+    output and all ten gradients against the oracle, bounded by the order-only floor measured on the same inputs."""
+    say("config", cfg, "full size against the oracle", b, L, d, dh, C)
+    inp = O.make_inputs(b, L, d, dh, seed=seed, act_dtype=torch.bfloat16, distinct_heads=4)
+    res, ref, floors = run_both(*block_causal_pair(C, True), inp, AC, floor=True)
+    if cfg == 1:
+        # nothing is carried into the only update: d loss / d momentum is exactly zero on both sides
+        assert float(res["momentum"].abs().max()) == 0.0 and float(ref["momentum"].abs().max()) == 0.0
+    assert_within_order_floor(res, ref, floors, f"config-{cfg}")
 
 
 def test_config1_full_size_properties():

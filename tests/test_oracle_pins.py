@@ -17,6 +17,7 @@ from oracle import lact_oracle as O
 
 torch.manual_seed(0)
 F64 = O.Numerics(autocast=False, ns_dtype=None)
+PLAIN = O.Numerics(autocast=False)
 GOLD = os.path.join(os.path.dirname(__file__), "golden", "bidirectional_muon_cpu_fp32.npz")
 
 
@@ -415,3 +416,48 @@ def test_order_only_floor_of_bf16_newton_schulz(b, L, d, dh, C):
             assert 3e-3 < f_out < 4e-2 and 3e-3 < f_w < 4e-2
         else:
             assert f_out < 1e-3 and f_w < 1e-4
+
+
+# ---- golden vectors of the LLM operations and the NVS program, written from the reference (CPU, fp32) ---------
+LLM_NVS_GOLD = os.path.join(os.path.dirname(__file__), "golden", "llm_nvs_cpu_fp32.npz")
+LLM_TAGS = ("llm_plain", "llm_momentum", "llm_muon", "llm_prenorm", "llm_prenorm_muon")
+NVS_TAGS = ("nvs_update_then_apply", "nvs_update_and_apply_muon", "nvs_two_updates_muon")
+
+
+def load_llm_nvs_gold(tag):
+    z = np.load(LLM_NVS_GOLD)
+    pick = lambda kind: {k.split(f".{kind}.")[1]: z[k] for k in z.files if k.startswith(f"{tag}.{kind}.")}
+    t = {n: torch.from_numpy(a) for n, a in pick("in").items()}
+    grads = {n: torch.from_numpy(a) for n, a in pick("grad").items()}
+    outs = [torch.from_numpy(a) for _, a in sorted(pick("out").items())]
+    gos = [torch.from_numpy(a) for _, a in sorted(pick("go").items())]
+    return t, outs, gos, grads, pick("meta")
+
+
+def run_oracle_on_gold(tag, t, meta, num=PLAIN):
+    t = {n: v.clone().requires_grad_(True) for n, v in t.items()}
+    a = [t[n] for n in ("w0", "w1", "w2", "q", "k", "v", "lr0", "lr1", "lr2")]
+    if tag.startswith("llm"):
+        res = [O.block_causal_lact_swiglu(*a, int(meta["chunk"]), bool(meta["use_muon"]), t.get("momentum"), num=num,
+                                          prenorm=bool(meta["prenorm"]))]
+    else:
+        order = [O.TTTOperator(int(s), int(e), bool(u), bool(ap)) for s, e, u, ap in meta["order"]]
+        res = list(O.fast_weight_swish_glu_weight_norm_mini_batch_apply(*a, order, int(meta["steps"]), num=num))
+    return t, res
+
+
+@pytest.mark.parametrize("tag", LLM_TAGS + NVS_TAGS)
+def test_llm_and_nvs_golden(tag):
+    """tests/golden/make_llm_nvs_golden.py: ttt_operation.py:71-364 and lact_ttt.py:71-147 themselves, run on the CPU:
+    output, returned weights and the gradient of every input.  Same library, same operations in the same order:
+    the oracle has to reproduce them to fp32 round-off, Newton-Schulz in bf16 included."""
+    t, outs, gos, grads, meta = load_llm_nvs_gold(tag)
+    tt, res = run_oracle_on_gold(tag, t, meta)
+    assert len(res) == len(outs)
+    for r, o in zip(res, outs):
+        assert r.shape == o.shape and O.rel_l2(r, o) < 1e-5, (tag, O.rel_l2(r, o))
+    loss = sum((r.float() * go).sum() for r, go in zip(res, gos))
+    names = list(grads)
+    got = torch.autograd.grad(loss, [tt[n] for n in names])
+    for n, g in zip(names, got):
+        assert O.rel_l2(g, grads[n]) < 1e-5, (tag, n, O.rel_l2(g, grads[n]))
