@@ -121,6 +121,13 @@ size_t lact_newton_schulz_workspace_bytes(int32_t n, int32_t rows, int32_t cols,
 int lact_newton_schulz(int32_t n, int32_t rows, int32_t cols, const float* g, float* out, int32_t steps,
                        const float* coeffs, int32_t ns_mode, void* workspace, void* stream);
 
+/* Backward of lact_newton_schulz (in the reference autograd differentiates ttt_operation.py:30-66 / lact_ttt.py:33-67):
+ * dg = d loss / d g from dout = d loss / d out; g, dout, dg: [n, rows, cols] fp32.  Recomputes the iterates from g (same
+ * steps, coeffs, ns_mode as the forward call), then walks them backwards in closed form. */
+size_t lact_newton_schulz_backward_workspace_bytes(int32_t n, int32_t rows, int32_t cols, int32_t steps);
+int lact_newton_schulz_backward(int32_t n, int32_t rows, int32_t cols, const float* g, const float* dout, float* dg,
+                                int32_t steps, const float* coeffs, int32_t ns_mode, void* workspace, void* stream);
+
 /* lact_newton_schulz for callers that cannot allocate device memory or hand over a workspace (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The workspace is
  * a fixed array of LACT_NS_STATIC_WORKSPACE_BYTES in device memory that the library holds on every GPU it runs on
@@ -184,6 +191,15 @@ int lact_layer_post_backward(int32_t act_dtype, int32_t B, int32_t L, int32_t H,
  * Returns the previous value (0 / 1, or the previous limit), or -1 for an unknown option. */
 enum { LACT_OPT_STREAM_OVERLAP = 0, LACT_OPT_FUSED_NEWTON_SCHULZ = 1, LACT_OPT_NS_BARRIER_SPIN_LIMIT = 2 };
 int lact_set_option(int32_t option, int32_t value);
+
+/* Errors that only the device notices.  A block of the fused Newton-Schulz kernel that gives up at a barrier (see
+ * LACT_OPT_NS_BARRIER_SPIN_LIMIT) turns the step's results into NaN and adds one to a per-device counter that no
+ * call clears.  lact_check_async_error copies that counter of the current device to the host (a synchronous copy: call
+ * it once the stream the steps ran on has been synchronised), resets it and returns it: 0 = nothing happened, > 0 =
+ * that many waits timed out since the last check (message in lact_last_error), < 0 = the check itself failed.  No
+ * counterpart in the reference, whose kernels never wait for each other.  The fused kernel is only used on a device
+ * with at least 256 compute units (its groups must be resident as a whole); elsewhere the unfused launches run. */
+int lact_check_async_error(void);
 
 /* Per-launch timing with HIP events on the caller's stream (no counterpart in the reference, which
  * times with wall-clock prints, lact_ar_video/minVid/train.py:458-460).  While enabled every kernel

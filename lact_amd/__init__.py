@@ -8,7 +8,7 @@ The package mirrors the reference's call signatures for this one path:
   lact_amd.layers         <- minimal_implementations/bidirectional_lact_layer.py, causal_lact_with_sliding_window_attn.py
                              (the two layer classes around the operation)
 All arithmetic runs in lib/liblact_hip.so (built from csrc/ with hipcc for gfx950)."""
-from .ops import NS5_COEFFS, NS_CLASSIC, Program, block_causal_steps, run_program  # noqa: F401
+from .ops import NS5_COEFFS, NS_CLASSIC, Program, block_causal_steps, check_async_error, run_program  # noqa: F401
 from .ttt_operation import (block_causal_lact_swiglu, l2_norm, prenorm_block_causal_lact_swiglu,  # noqa: F401
                             postnorm_block_causal_lact_swiglu_fused_kernel_triton,
                             prenorm_block_causal_lact_swiglu_fused_kernel_triton,

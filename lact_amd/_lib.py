@@ -37,7 +37,8 @@ class Desc(Structure):
 OPT_STREAM_OVERLAP, OPT_FUSED_NEWTON_SCHULZ, OPT_NS_BARRIER_SPIN_LIMIT = 0, 1, 2
 EXPORTS = ("lact_last_error", "lact_version", "lact_query_sizes", "lact_forward", "lact_forward_from_state", "lact_backward",
            "lact_newton_schulz_workspace_bytes", "lact_newton_schulz", "lact_newton_schulz_static_capacity",
-           "lact_newton_schulz_static", "lact_set_option", "lact_profile_enable",
+           "lact_newton_schulz_static", "lact_newton_schulz_backward_workspace_bytes", "lact_newton_schulz_backward",
+           "lact_check_async_error", "lact_set_option", "lact_profile_enable",
            "lact_profile_report", "lact_layer_pre_forward", "lact_layer_pre_backward", "lact_layer_lr_forward",
            "lact_layer_lr_backward", "lact_layer_post_forward", "lact_layer_post_dw_rows", "lact_layer_post_backward")
 
@@ -72,6 +73,12 @@ def lib():
     L.lact_newton_schulz_static_capacity.restype = c_size_t
     L.lact_newton_schulz_static.argtypes = [c_int32, c_int32, c_int32, vp, vp, c_int32, POINTER(c_float), c_int32, vp]
     L.lact_newton_schulz_static.restype = c_int32
+    L.lact_newton_schulz_backward_workspace_bytes.argtypes = [c_int32] * 4
+    L.lact_newton_schulz_backward_workspace_bytes.restype = c_size_t
+    L.lact_newton_schulz_backward.argtypes = [c_int32, c_int32, c_int32, vp, vp, vp, c_int32, POINTER(c_float), c_int32, vp, vp]
+    L.lact_newton_schulz_backward.restype = c_int32
+    L.lact_check_async_error.argtypes = []
+    L.lact_check_async_error.restype = c_int32
     L.lact_set_option.argtypes = [c_int32, c_int32]
     L.lact_set_option.restype = c_int32
     i32, f32 = c_int32, c_float

@@ -124,6 +124,8 @@ struct SideCtx {
   size_t next = 0;
   hipEvent_t fused_done = nullptr;   // completion of the newest fused Newton-Schulz kernel of this process
   bool fused_recorded = false;
+  int cus = 0;                       // compute units of the device (0: not asked yet)
+  unsigned* sticky = nullptr;        // device address of this device's count of barrier time-outs
   hipEvent_t event() {
     if (next == ev.size()) {
       hipEvent_t e;
@@ -133,6 +135,11 @@ struct SideCtx {
     return ev[next++];
   }
 };
+}  // namespace
+// Barrier waits of the fused Newton-Schulz kernels that gave up, counted per device since the last
+// lact_check_async_error (each GPU holds its own copy; host code reaches it through hipGetSymbolAddress only).
+static __device__ unsigned g_async_errors;
+namespace {
 bool g_overlap = true;
 bool g_fused_ns = true;
 long long g_ns_spin_limit = NS_FUSED_SPIN_LIMIT;   // barrier wait bound of the fused Newton-Schulz kernels (lact_set_option)
@@ -144,6 +151,14 @@ SideCtx* side_ctx() {
   SideCtx& c = ctx[dev];
   if (!c.stream && hipStreamCreateWithFlags(&c.stream, hipStreamNonBlocking) != hipSuccess) return nullptr;
   if (!c.tail && hipStreamCreateWithFlags(&c.tail, hipStreamNonBlocking) != hipSuccess) return nullptr;
+  if (c.cus == 0) {
+    int n = 0;
+    c.cus = (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) ? n : -1;
+  }
+  if (!c.sticky) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_async_errors)) == hipSuccess) c.sticky = static_cast<unsigned*>(ptr);
+  }
   c.next = 0;
   return &c;
 }
@@ -516,8 +531,11 @@ struct Runner {
       default: return 0;
     }
   }
+  // The fused kernel's groups must be resident as a whole, one block per compute unit, on a device that deals its
+  // workgroups to 8 dies of 32 compute units: anything else (a partitioned or smaller device) takes the unfused launches.
   bool ns_fused_ok(const NsBatch& B) const {
     if (!g_fused_ns || !side || !kNsBf16 || P.S < 1 || P.S > NS_FUSED_MAX_STEPS) return false;
+    if (side->cus < 256) return false;
     return ns_fused_tile(B) >= 0;
   }
   // every batch runs fused (and at least one iteration): the Frobenius normalisation is the fused kernel's first stage
@@ -550,6 +568,7 @@ struct Runner {
     p.r = B.r; p.c = B.c; p.S = P.S; p.nb = B.nb; p.mask = B.mask;
     for (int i = 0; i < 3 * P.S; ++i) p.coeffs[i] = P.coeffs[i];
     p.error = ns_error_word();
+    p.sticky = side->sticky;
     p.spin_limit = g_ns_spin_limit;
     const double terms = BWD ? 6.0 : 3.0;
     static const std::string name = std::string("k_ns_fused<") + std::to_string(TS::BM) + "x" + std::to_string(TS::BN) + (BWD ? ",bwd>" : ",fwd>");
@@ -1616,6 +1635,119 @@ int newton_schulz_t(int32_t n, int32_t rows, int32_t cols, const float* gin, flo
 }  // namespace
 
 
+// ---- backward of the standalone Newton-Schulz: recomputes the iterates, then walks them backwards ------------
+namespace {
+struct NsBwdPlan {
+  NsPlan f;
+  size_t o_xb, o_ab, o_bb, o_gxf[2], o_gxb[2], o_sg, o_gas, o_dot, bytes;
+  void build(int n, int rows, int cols, int steps) {
+    f.build(n, rows, cols);
+    Bump b;
+    b.off = f.bytes;
+    const size_t e = (size_t)n * f.g.elems, sq = (size_t)n * f.r * f.r, S = (size_t)std::max(1, steps);
+    o_xb = b.take(S * e * 4); o_ab = b.take(S * sq * 4); o_bb = b.take(S * sq * 4);
+    for (int i = 0; i < 2; ++i) { o_gxf[i] = b.take(e * 4); o_gxb[i] = b.take(e * 4); }
+    o_sg = b.take(sq * 4); o_gas = b.take(sq * 4); o_dot = b.take((size_t)n * f.nblk * 4);
+    bytes = b.off + 256;
+  }
+};
+
+template <typename TN>
+int newton_schulz_bwd_t(int32_t n, int32_t rows, int32_t cols, const float* gin, const float* dout, float* dg, int32_t steps,
+                        const float* coeffs, int32_t ns_mode, void* workspace, hipStream_t s) {
+  const int plain_bf16 = ns_mode == LACT_NS_PLAIN_BF16;
+  NsBwdPlan P;
+  P.build(n, rows, cols, steps);
+  const NsPlan& F = P.f;
+  char* ws = align256(workspace);
+  const size_t e = (size_t)n * F.g.elems, sq = (size_t)n * F.r * F.r;
+  auto xb = [&](int it) { return reinterpret_cast<TN*>(ws + P.o_xb) + (size_t)it * e; };
+  auto ab = [&](int it) { return reinterpret_cast<TN*>(ws + P.o_ab) + (size_t)it * sq; };
+  auto bb = [&](int it) { return reinterpret_cast<TN*>(ws + P.o_bb) + (size_t)it * sq; };
+  // ---- forward again, keeping X_k, A_k, B_k
+  MomentumPrepParams mp;
+  memset(&mp, 0, sizeof(mp));
+  mp.g = F.g; mp.partial = gin; mp.nsplit = 1; mp.d_out = nullptr;
+  mp.g16 = ws + F.o_g16; mp.ss_part = reinterpret_cast<float*>(ws + F.o_ss);
+  LACT_LAUNCH("k_momentum_prep", "k_momentum_prep", 0.0, (k_momentum_prep<TN>), dim3(F.nblk, n), dim3(256), s, mp);
+  NsScaleParams sp;
+  memset(&sp, 0, sizeof(sp));
+  sp.g = F.g; sp.g16 = mp.g16; sp.ss_part = mp.ss_part; sp.nparts = F.nblk; sp.norms = reinterpret_cast<float*>(ws + F.o_norm);
+  sp.xf = reinterpret_cast<float*>(ws + F.o_xf[0]); sp.xb = xb(0); sp.plain_bf16 = plain_bf16;
+  LACT_LAUNCH("k_ns_scale", "k_ns_scale", 0.0, (k_ns_scale<TN>), dim3(F.nblk, n), dim3(256), s, sp);
+  for (int it = 0; it + 1 < steps; ++it) {   // the last iterate itself is not needed
+    NsIter I;
+    I.n = n; I.r = F.r; I.c = F.c; I.nb_for_mask = n; I.mask = 0; I.plain = plain_bf16;
+    I.ca = coeffs[3 * it]; I.cb = coeffs[3 * it + 1]; I.cc = coeffs[3 * it + 2];
+    I.xf_in = reinterpret_cast<float*>(ws + F.o_xf[it & 1]); I.xb_in = xb(it);
+    I.ab = ab(it); I.bb = bb(it); I.cab = ws + F.o_ca;
+    I.xf_out = reinterpret_cast<float*>(ws + F.o_xf[(it + 1) & 1]); I.xb_out = xb(it + 1); I.u_out = nullptr;
+    ns_iteration<TN>(I, s);
+  }
+  if (steps > 0) {   // A and B of the last iteration (its X' is the output the caller already has)
+    const int it = steps - 1;
+    const long long xe = (long long)F.r * F.c, se = (long long)F.r * F.r;
+    auto p = row_params<1>();
+    set_term(p.t[0], xb(it), F.c, xe, xb(it), F.c, xe, F.c);
+    p.M = F.r; p.N = F.r; p.out = ab(it); p.ldo = F.r; p.bso = se;
+    p.out2 = ws + F.o_ca; p.alpha2 = coeffs[3 * it + 2];
+    launch_row_gemm<TN, true, 1, EPI_STORE>("ns_gram", p, n, s);
+    auto q = row_params<1>();
+    set_term(q.t[0], ws + F.o_ca, F.r, se, ab(it), F.r, se, F.r);
+    q.M = F.r; q.N = F.r; q.out = bb(it); q.ldo = F.r; q.bso = se;
+    q.aux = ab(it); q.ldaux = F.r; q.bsaux = se; q.alpha = 1.f; q.beta = coeffs[3 * it + 1];
+    launch_row_gemm<TN, true, 1, EPI_AXPBY>("ns_poly", q, n, s);
+  }
+  // ---- the incoming gradient where Newton-Schulz holds its matrices
+  float* gxf[2] = {reinterpret_cast<float*>(ws + P.o_gxf[0]), reinterpret_cast<float*>(ws + P.o_gxf[1])};
+  TN* gxb[2] = {reinterpret_cast<TN*>(ws + P.o_gxb[0]), reinterpret_cast<TN*>(ws + P.o_gxb[1])};
+  LACT_LAUNCH("k_to_ns_orientation", "k_to_ns_orientation", 0.0, (k_to_ns_orientation<TN>), dim3(F.nblk, n), dim3(256), s, F.g, dout, gxf[0], (void*)gxb[0]);
+  TN* sg = reinterpret_cast<TN*>(ws + P.o_sg);
+  TN* gas = reinterpret_cast<TN*>(ws + P.o_gas);
+  const long long xe = (long long)F.r * F.c, se = (long long)F.r * F.r;
+  int bc = 0;
+  for (int it = steps - 1; it >= 0; --it) {
+    const float ca = coeffs[3 * it], cb = coeffs[3 * it + 1], cc = coeffs[3 * it + 2];
+    {  // Sg = G X^T + X G^T
+      auto p = row_params<2>();
+      set_term(p.t[0], gxb[bc], F.c, xe, xb(it), F.c, xe, F.c);
+      set_term(p.t[1], xb(it), F.c, xe, gxb[bc], F.c, xe, F.c);
+      p.M = F.r; p.N = F.r; p.out = sg; p.ldo = F.r; p.bso = se;
+      launch_row_gemm<TN, true, 2, EPI_STORE>("ns_bwd_sg", p, n, s);
+    }
+    {  // gA + gA^T = b Sg + c (Sg A + A Sg)
+      auto p = row_params<2>();
+      set_term(p.t[0], sg, F.r, se, ab(it), F.r, se, F.r);
+      set_term(p.t[1], ab(it), F.r, se, sg, F.r, se, F.r);
+      p.M = F.r; p.N = F.r; p.out = gas; p.ldo = F.r; p.bso = se;
+      p.aux = sg; p.ldaux = F.r; p.bsaux = se; p.alpha = cc; p.beta = cb;
+      launch_row_gemm<TN, true, 2, EPI_AXPBY>("ns_bwd_ga", p, n, s);
+    }
+    {  // gX = a G + B G + (gA + gA^T) X
+      auto p = row_params<2>();
+      set_term(p.t[0], bb(it), F.r, se, gxb[bc], F.c, xe, F.r);
+      set_term(p.t[1], gas, F.r, se, xb(it), F.c, xe, F.r);
+      p.M = F.r; p.N = F.c; p.ldo = F.c; p.bso = xe;
+      p.aux = gxf[bc]; p.ldaux = F.c; p.bsaux = xe; p.alpha = 1.f; p.beta = ca;
+      p.out = gxf[bc ^ 1]; p.out_c = gxb[bc ^ 1];
+      launch_row_gemm<TN, false, 2, EPI_AXPBY_F32_DUAL>("ns_bwd_gx", p, n, s);
+    }
+    bc ^= 1;
+  }
+  // ---- backward of X0 = G16 / (|G16| + 1e-7) and of the cast
+  NsDotParams dp;
+  dp.g = F.g; dp.gx0 = gxf[bc]; dp.g16 = ws + F.o_g16; dp.dot_part = reinterpret_cast<float*>(ws + P.o_dot);
+  LACT_LAUNCH("k_ns_bwd_dot", "k_ns_bwd_dot", 0.0, (k_ns_bwd_dot<TN>), dim3(F.nblk, n), dim3(256), s, dp);
+  GradPrepParams gp;
+  memset(&gp, 0, sizeof(gp));
+  gp.g = F.g; gp.muon = 1; gp.gx0 = gxf[bc]; gp.g16 = ws + F.o_g16; gp.norms = reinterpret_cast<float*>(ws + F.o_norm);
+  gp.dot_part = dp.dot_part; gp.nparts = F.nblk; gp.gc = dg;
+  LACT_LAUNCH("k_grad_prep", "k_grad_prep", 0.0, (k_grad_prep<float, TN>), dim3(F.nblk, n), dim3(256), s, gp);
+  LACT_CHECK_LAUNCH();
+  return 0;
+}
+}  // namespace
+
 // ---- Newton-Schulz without a caller workspace: the workspace is a fixed array in device memory -------------
 // Every GPU the library runs on holds its own copy of the array (at its own address) until the process ends.
 // In host code the array's name is only a handle for hipGetSymbolAddress; the address it returns for the current
@@ -1781,6 +1913,19 @@ int lact_layer_post_backward(int32_t act_dtype, int32_t B, int32_t L, int32_t H,
   return 0;
 }
 
+int lact_check_async_error(void) {
+  unsigned n = 0;
+  hipError_t e = hipMemcpyFromSymbol(&n, HIP_SYMBOL(g_async_errors), sizeof(n), 0, hipMemcpyDeviceToHost);
+  if (e != hipSuccess) return fail(std::string("lact_check_async_error: ") + hipGetErrorString(e));
+  if (n == 0) return 0;
+  const unsigned zero = 0;
+  (void)hipMemcpyToSymbol(HIP_SYMBOL(g_async_errors), &zero, sizeof(zero), 0, hipMemcpyHostToDevice);
+  g_err = std::to_string(n) + " barrier wait(s) of the fused Newton-Schulz kernel timed out on this device since the last check: "
+          "the results of those steps are NaN (compute units held by another process or kernel; raise "
+          "LACT_OPT_NS_BARRIER_SPIN_LIMIT or switch LACT_OPT_FUSED_NEWTON_SCHULZ off)";
+  return (int)std::min<unsigned>(n, 0x7fffffffu);
+}
+
 int lact_profile_enable(int on) {
   g_prof.clear();
   g_prof.on = on != 0;
@@ -1909,6 +2054,25 @@ int lact_newton_schulz(int32_t n, int32_t rows, int32_t cols, const float* gin, 
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (ns_mode == LACT_NS_FP32) return newton_schulz_t<float>(n, rows, cols, gin, out, steps, coeffs, ns_mode, workspace, s);
   return newton_schulz_t<uint16_t>(n, rows, cols, gin, out, steps, coeffs, ns_mode, workspace, s);
+}
+
+size_t lact_newton_schulz_backward_workspace_bytes(int32_t n, int32_t rows, int32_t cols, int32_t steps) {
+  if (n <= 0 || rows <= 0 || cols <= 0 || steps < 0) return 0;
+  NsBwdPlan P;
+  P.build(n, rows, cols, steps);
+  return P.bytes;
+}
+
+int lact_newton_schulz_backward(int32_t n, int32_t rows, int32_t cols, const float* gin, const float* dout, float* dg,
+                                int32_t steps, const float* coeffs, int32_t ns_mode, void* workspace, void* stream) {
+  if (n <= 0 || rows <= 0 || cols <= 0 || n > 65535) return fail("bad Newton-Schulz shape");
+  if (rows % 8 || cols % 8) return fail("rows and cols must be multiples of 8");
+  if (steps < 0 || steps > 64 || (steps > 0 && !coeffs)) return fail("bad Newton-Schulz steps");
+  if (ns_mode < 0 || ns_mode > 2) return fail("ns_mode must be 0, 1 or 2");
+  if (!gin || !dout || !dg || !workspace) return fail("null pointer: newton_schulz_backward");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (ns_mode == LACT_NS_FP32) return newton_schulz_bwd_t<float>(n, rows, cols, gin, dout, dg, steps, coeffs, ns_mode, workspace, s);
+  return newton_schulz_bwd_t<uint16_t>(n, rows, cols, gin, dout, dg, steps, coeffs, ns_mode, workspace, s);
 }
 
 size_t lact_newton_schulz_static_capacity(void) { return LACT_NS_STATIC_WORKSPACE_BYTES; }

@@ -64,16 +64,18 @@ struct NsFusedParams {
   const float* m_prev; const float* mbar; float* mdot_part;
   unsigned* sync;            // [n][32] words, zeroed before the launch: word 0 = arrivals, word 1 = XCC id mask
   unsigned* error;           // set to 1 by a block whose barrier timed out
+  unsigned* sticky;          // per-device count of such time-outs (not cleared between calls), or null
   long long spin_limit;      // polls a block waits at a barrier before it gives up
 };
 
 struct GroupBarrier {
   unsigned* ctr;
+  unsigned* sticky;          // per-device count of timed-out waits, never cleared by a kernel (lact_check_async_error reads it)
   unsigned members, epoch;
   long long limit;
   bool split;                // group spread over several XCDs: fence at device scope
-  __device__ __forceinline__ void init(unsigned* line, unsigned nmembers, unsigned* error, long long spin_limit) {
-    ctr = line; members = nmembers; epoch = 0; split = false; limit = spin_limit;
+  __device__ __forceinline__ void init(unsigned* line, unsigned nmembers, unsigned* error, long long spin_limit, unsigned* sticky_count) {
+    ctr = line; members = nmembers; epoch = 0; split = false; limit = spin_limit; sticky = sticky_count;
     unsigned xcc = 0;
     asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
     if (threadIdx.x == 0) __hip_atomic_fetch_or(line + 1, 1u << (xcc & 0xf), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -83,7 +85,11 @@ struct GroupBarrier {
   }
   // all threads of the block call it
   __device__ __forceinline__ void sync(unsigned* error, bool heavy = false) {
-    __syncthreads();   // every wave has waited for its stores before it gets here
+    // Every wave waits for its own stores of the stage: a store that has been waited for is in this XCD's L2 (the
+    // vector L1 writes through), which is where the partner blocks' device-scope loads look.  Without the wait the
+    // arrival below could overtake a store that is still on its way to another L2 channel.
+    wait_vmcnt<0>();
+    __syncthreads();
     if (threadIdx.x == 0) {
       const bool fence = heavy || split;
       if (fence) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
@@ -94,6 +100,7 @@ struct GroupBarrier {
         __builtin_amdgcn_s_sleep(1);
         if (++spins > limit) {
           __hip_atomic_store(error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (sticky) __hip_atomic_fetch_add(sticky, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           break;
         }
       }
@@ -131,7 +138,7 @@ __global__ __launch_bounds__(DMA_THREADS) void k_ns_fused(const NsFusedParams p)
   if (group >= p.n) return;
   const int z = p.z0 + group;
   GroupBarrier bar;
-  bar.init(p.sync + (size_t)group * 32, nbm, p.error, p.spin_limit);
+  bar.init(p.sync + (size_t)group * 32, nbm, p.error, p.spin_limit, p.sticky);
   const bool sq_tile = member < tr * ts;             // this block owns a tile of the r x r stages
   const int sx = member / ts, sy = member % ts;      // its tile there
   const int rx = member / tc, ry = member % tc;      // its tile of the r x c stages
@@ -268,7 +275,9 @@ __global__ __launch_bounds__(DMA_THREADS) void k_ns_fused(const NsFusedParams p)
     float4 ga[NG], gb[NG];
     uint4 gi[NG];
     float dot = 0.f;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");   // the vector L1 may hold this buffer's lines from two iterations ago
+    // No fence: this tile of gx was written by this very block in the last stage (and in every second stage before),
+    // and the waves of a compute unit share its vector L1, which their own stores keep current.  The same holds for
+    // every auxiliary tile the blending epilogues read (always the block's own tile of a buffer it wrote itself).
 #pragma unroll
     for (int t = 0; t < NG; ++t) {
       const int id = threadIdx.x + t * DMA_THREADS;

@@ -401,6 +401,32 @@ __global__ void k_renorm_bwd(const RenormParams p) {
     emit(c, renorm_gy4(p, o + c), p.weight_norm ? renorm_w_hat4(p, o + c, uo + c) : zero4);
 }
 
+// A gradient given in the original orientation of its matrices, copied to where Newton-Schulz holds them (fp32 and
+// Newton-Schulz type).  Grid (chunks, matrices).
+template <typename TN>
+__global__ void k_to_ns_orientation(const MatGeom g, const float* in, float* xf, void* xb) {
+  const int z = blockIdx.y, j = z / g.nb;
+  const FlatRange R(g.elems);
+  const size_t zo = (size_t)z * g.elems, xo = g.ns_base(g.ns_of(z));
+  const bool contiguous = g.x_contiguous(j);
+  for (long long e = R.e0 + threadIdx.x * 4; e < R.e1; e += blockDim.x * 4) {
+    const float4 v = ld4(in + zo + e);
+    if (contiguous) {
+      const size_t x = xo + g.xidx(j, e);
+      st4(xf + x, v);
+      Elem<TN>::store4(reinterpret_cast<TN*>(xb) + x, v.x, v.y, v.z, v.w);
+    } else {
+      const float a[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const size_t x = xo + g.xidx(j, e + i);
+        xf[x] = a[i];
+        Elem<TN>::store(reinterpret_cast<TN*>(xb) + x, a[i]);
+      }
+    }
+  }
+}
+
 // ---- backward of the Frobenius normalisation, the momentum recurrence and the raw-gradient add --
 struct NsDotParams {
   MatGeom g;

@@ -141,7 +141,7 @@ def _covers(steps, out_len: int) -> bool:
 
 class _LactProgramFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, prog: Program, w0, w1, w2, q, k, v, lr0, lr1, lr2, momentum, m_state=None):
+    def forward(ctx, prog: Program, w0, w1, w2, q, k, v, lr0, lr1, lr2, momentum, m_state=None, grad_mode=True):
         if not q.is_cuda:
             raise RuntimeError("lact_amd runs on an MI355X only: tensors must be on a HIP device (no CPU path)")
         L = _lib.lib()
@@ -163,7 +163,9 @@ class _LactProgramFn(torch.autograd.Function):
         out = alloc((b, prog.out_len, d), dtype=act, device=q.device)
         call = _Call(prog, b, d, dh, qa, ka, va, out)
         call.desc.use_momentum = int(mom is not None)
-        call.desc.forward_only = int(not any(ctx.needs_input_grad))
+        # needs_input_grad ignores the grad mode (and inside forward grad mode is always off): the caller's mode
+        # comes in as an argument -- under torch.no_grad() nothing will ask for a backward pass
+        call.desc.forward_only = int(not (grad_mode and any(ctx.needs_input_grad)))
         m_in = None
         if m_state is not None and mom is not None:
             if not call.desc.forward_only:
@@ -240,14 +242,14 @@ class _LactProgramFn(torch.autograd.Function):
         glr = [None if g is None else g.reshape(lr_shape).to(ctx.lr_dtype) for g in dlr]
         gm = None if dmom is None else dmom.reshape(mom_shape).to(ctx.mom_dtype)
         return (None, cast(dw[0], wd0), cast(dw[1], wd1), cast(dw[2], wd2), cast(dq, qd), cast(dk, kd), cast(dv, vd),
-                glr[0], glr[1], glr[2], gm, None)
+                glr[0], glr[1], glr[2], gm, None, None)
 
 
 @torch.compiler.disable
 def run_program(prog: Program, w0, w1, w2, q, k, v, lr0, lr1, lr2, momentum=None, momentum_state=None):
     """Runs `prog`.  Returns (out, (w0, w1, w2) after the last update, (m0, m1, m2) momentum states).
     `momentum_state` = the (m0, m1, m2) of an earlier call: the first update continues from it (inference only)."""
-    res = _LactProgramFn.apply(prog, w0, w1, w2, q, k, v, lr0, lr1, lr2, momentum, momentum_state)
+    res = _LactProgramFn.apply(prog, w0, w1, w2, q, k, v, lr0, lr1, lr2, momentum, momentum_state, torch.is_grad_enabled())
     return res[0], res[1:4], res[4:7]
 
 
@@ -281,23 +283,57 @@ def _ns_mode(q: torch.Tensor) -> int:
     return NS_PLAIN_BF16 if (q.dtype == torch.float32 and not torch.is_autocast_enabled()) else NS_AUTOCAST
 
 
+class _NewtonSchulzFn(torch.autograd.Function):
+    """zeropower_via_newtonschulz5 with its closed-form backward (lact_newton_schulz / lact_newton_schulz_backward)."""
+
+    @staticmethod
+    def forward(ctx, G, coeffs, ns_mode):
+        L = _lib.lib()
+        n, rows, cols = G.shape
+        g = G.detach().float().contiguous()
+        out = torch.empty_like(g)
+        ws = torch.empty(L.lact_newton_schulz_workspace_bytes(n, rows, cols, len(coeffs)), dtype=torch.uint8, device=G.device)
+        flat = [float(x) for tr in coeffs for x in tr]
+        arr = (ctypes.c_float * max(1, len(flat)))(*flat)
+        stream = ctypes.c_void_p(torch.cuda.current_stream(G.device).cuda_stream)
+        with torch.cuda.device(G.device):
+            _lib.check(L.lact_newton_schulz(n, rows, cols, _ptr(g), _ptr(out), len(coeffs), arr, int(ns_mode), _ptr(ws), stream))
+        ctx.save_for_backward(g)
+        ctx.coeffs, ctx.ns_mode, ctx.in_dtype = tuple(coeffs), int(ns_mode), G.dtype
+        return out.to(torch.bfloat16) if ns_mode == NS_PLAIN_BF16 else out
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, dout):
+        (g,) = ctx.saved_tensors
+        L = _lib.lib()
+        n, rows, cols = g.shape
+        do = dout.detach().float().contiguous()
+        dg = torch.empty_like(g)
+        steps = len(ctx.coeffs)
+        ws = torch.empty(L.lact_newton_schulz_backward_workspace_bytes(n, rows, cols, steps), dtype=torch.uint8, device=g.device)
+        flat = [float(x) for tr in ctx.coeffs for x in tr]
+        arr = (ctypes.c_float * max(1, len(flat)))(*flat)
+        stream = ctypes.c_void_p(torch.cuda.current_stream(g.device).cuda_stream)
+        with torch.cuda.device(g.device):
+            _lib.check(L.lact_newton_schulz_backward(n, rows, cols, _ptr(g), _ptr(do), _ptr(dg), steps, arr, ctx.ns_mode, _ptr(ws), stream))
+        return dg.to(ctx.in_dtype), None, None
+
+
 @torch.compiler.disable
 def newton_schulz(G: torch.Tensor, coeffs: Sequence[Tuple[float, float, float]], ns_mode: int = NS_PLAIN_BF16) -> torch.Tensor:
-    """zeropower_via_newtonschulz5 on [n, rows, cols]; forward only."""
+    """zeropower_via_newtonschulz5 on [n, rows, cols] (ttt_operation.py:30-66; lact_ttt.py:33-67), differentiable."""
     if G.dim() != 3:
         raise AssertionError("expected a 3-D tensor")          # ttt_operation.py:44
     if not G.is_cuda:
         raise RuntimeError("lact_amd runs on an MI355X only (no CPU path)")
-    if G.requires_grad and torch.is_grad_enabled():
-        raise RuntimeError("standalone newton_schulz is forward-only; differentiate through run_program instead")
-    L = _lib.lib()
-    n, rows, cols = G.shape
-    g = G.detach().float().contiguous()
-    out = torch.empty_like(g)
-    ws = torch.empty(L.lact_newton_schulz_workspace_bytes(n, rows, cols, len(coeffs)), dtype=torch.uint8, device=G.device)
-    flat = [float(x) for tr in coeffs for x in tr]
-    arr = (ctypes.c_float * max(1, len(flat)))(*flat)
-    stream = ctypes.c_void_p(torch.cuda.current_stream(G.device).cuda_stream)
-    with torch.cuda.device(G.device):
-        _lib.check(L.lact_newton_schulz(n, rows, cols, _ptr(g), _ptr(out), len(coeffs), arr, int(ns_mode), _ptr(ws), stream))
-    return out.to(torch.bfloat16) if ns_mode == NS_PLAIN_BF16 else out
+    return _NewtonSchulzFn.apply(G, tuple(tuple(c) for c in coeffs), int(ns_mode))
+
+
+def check_async_error() -> None:
+    """Raises if a barrier wait of the fused Newton-Schulz kernel timed out on the current device since the last check
+    (the results of those steps are NaN).  Synchronises the device; call it at a point where the host waits anyway."""
+    torch.cuda.synchronize()
+    n = _lib.lib().lact_check_async_error()
+    if n != 0:
+        raise RuntimeError("liblact_hip: " + _lib.lib().lact_last_error().decode())

@@ -162,6 +162,58 @@ def test_newton_schulz_standalone(n, r, c, kind, steps):
         assert e_ref <= 1.5 * floor + 1e-3
 
 
+@pytest.mark.parametrize("n,r,c,kind,steps", [(3, 64, 64, "llm", 5), (2, 128, 256, "llm", 5), (2, 256, 128, "classic", 3),
+                                              (2, 384, 384, "llm", 5), (2, 40, 24, "classic", 2), (2, 64, 128, "classic", 0)])
+def test_newton_schulz_standalone_is_differentiable(n, r, c, kind, steps):
+    """zeropower_via_newtonschulz5 is an ordinary differentiable function in the reference (ttt_operation.py:30-66):
+    lact_newton_schulz_backward against autograd through the oracle.  fp32 mode against float64 pins the closed form;
+    the reference's numerics are held to the larger of the order-only floor and the oracle's own distance from
+    float64 (the closed-form backward rounds at other points than autograd does: another realisation of the same
+    bf16 noise)."""
+    say("newton_schulz backward", n, r, c, kind, steps)
+    gen = torch.Generator().manual_seed(23)
+    G, go = torch.randn(n, r, c, generator=gen), torch.randn(n, r, c, generator=gen)
+    co = O.ns_coeff_table(kind, steps)
+
+    def oracle_grad(num, dt):
+        x = G.to(dt).requires_grad_(True)
+        y = O.newton_schulz(x, co, num)
+        return torch.autograd.grad(y, x, go.to(y.dtype))[0]
+
+    def hip_grad(mode):
+        x = G.to(DEV).requires_grad_(True)
+        y = ops.newton_schulz(x, co, ns_mode=mode)
+        return torch.autograd.grad(y, x, go.to(DEV).to(y.dtype))[0]
+    g64 = oracle_grad(EXACT, torch.float64)
+    e = O.rel_l2(hip_grad(ops.NS_FP32), g64)
+    say("   fp32 mode vs float64:", e)
+    assert e < 1e-3
+    for label, num, mode in (("autocast", AC, ops.NS_AUTOCAST), ("plain", PLAIN, ops.NS_PLAIN_BF16)):
+        ref = oracle_grad(num, torch.float32)
+        yard = max([O.rel_l2(ref, g64)] + [O.rel_l2(oracle_grad(v, torch.float32), ref) for v in O.order_variants(num)])
+        e = O.rel_l2(hip_grad(mode), ref)
+        say(f"   {label}: vs oracle {e:.4f}  yardstick {yard:.4f}")
+        assert e <= 1.5 * yard + 1e-3
+
+
+def test_no_grad_with_parameters_runs_the_inference_descriptor():
+    """Under torch.no_grad() inputs that require a gradient (nn.Parameter fast weights) still make autograd report
+    needs_input_grad; the call must all the same take the forward-only path -- smaller buffers, and the carried
+    momentum state (an inference feature) accepted."""
+    say("no_grad with requires_grad inputs")
+    inp = problem(2, 3 * 64, 64, 128, 31, torch.bfloat16, momentum=True)
+    g = clone_to(inp, DEV)                                    # every tensor requires a gradient
+    prog = ops.Program(steps=ops.block_causal_steps(3 * 64, 64), out_len=3 * 64, ns_coeffs=O.NS5_COEFFS)
+    with torch.no_grad():
+        out, ws, ms = ops.run_program(prog, *args9(g), g["momentum"])
+        M = [m.clone() for m in ms]
+        out2, _, ms2 = ops.run_program(prog, *args9(g), g["momentum"], momentum_state=M)     # raised before the fix
+    assert not out.requires_grad and torch.isfinite(out.float()).all() and torch.isfinite(out2.float()).all()
+    ref, _, _ = ops.run_program(prog, *args9(g), g["momentum"])                              # training descriptor
+    assert ref.requires_grad and torch.equal(ref.detach(), out)
+    assert not torch.equal(ms2[0], ms[0])                     # the carried state was used
+
+
 def block_causal_pair(C, use_muon, prenorm=False):
     fn = T.prenorm_block_causal_lact_swiglu if prenorm else T.block_causal_lact_swiglu
     hip = lambda t: fn(*args9(t), C, use_muon, t["momentum"])
@@ -664,12 +716,17 @@ def test_fused_newton_schulz_barrier_timeout_ends_every_kernel_and_poisons_the_s
     good_out, good = run()
     assert torch.isfinite(good_out).all()
     L = _lib.lib()
+    assert L.lact_check_async_error() == 0                     # nothing timed out so far in this process
     prev = L.lact_set_option(_lib.OPT_NS_BARRIER_SPIN_LIMIT, 1)
     try:
         assert prev > 1
         bad_out, bad = run()
     finally:
         assert L.lact_set_option(_lib.OPT_NS_BARRIER_SPIN_LIMIT, 0) == 1
+    # the time-outs reach the host: a count and a message, once
+    with pytest.raises(RuntimeError, match="timed out"):
+        ops.check_async_error()
+    assert L.lact_check_async_error() == 0
     assert torch.equal(bad_out[:, :128], good_out[:, :128])      # first chunk: initial weights, no Newton-Schulz yet
     assert torch.isnan(bad_out[:, 128:]).all()                   # everything behind the first update
     assert torch.isnan(bad["w0"]).all() and torch.isnan(bad["k"][:, :128]).all()
