@@ -35,23 +35,48 @@ CONFIGS = {
 }
 
 
-# HBM bytes per launch at config 1 (read + write), from the FETCH_SIZE / WRITE_SIZE counters of two
-# `rocprofv3 --pmc` runs scaled by a 1 GiB copy (profiles/c1_fwd_bwd_hbm_traffic_pmc.txt); MiB.
-MEASURED_TRAFFIC_MIB = {
-    "k_ns_fused<192x192,bwd>": 749.1 + 344.4,
-    "k_ns_fused<192x192,fwd>": 435.2 + 373.6,
-    "k_token_reduce_dma<192x192>": 120.3 + 22.5,
-    "k_token_reduce_rows_dma<192x192>": 355.6 + 75.0,
-    "k_update_bwd_hidden_kept_dma": 151.8 + 74.2,
-    "k_apply_bwd_hidden_dma": 77.9 + 72.0,
-    "k_update_hidden_dma": 79.1 + 144.0,
-    "k_apply_hidden_dma": 33.2 + 24.0,
-}
-
-
-# Whole step at config 1, same two counter runs (last line of that profile): read + written MiB
-MEASURED_STEP_TRAFFIC_MIB = 2792.0 + 1565.0
 PEAK_HBM_GBPS = 8000.0
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "{cfg}_fwd_bwd_hbm_traffic_pmc.txt")
+
+
+def _library_label(profile_name):
+    """Kernel name as rocprofv3 prints it (demangled) -> the label the library's own launch records use."""
+    import re
+    n = profile_name.strip()
+    n = re.sub(r"^void\s+", "", n).split("(")[0].replace("lact::", "")
+    n = re.sub(r"TileShape<(\d+), (\d+), \d+, \d+>\s*", r"\1x\2", n).replace(" ", "")
+    m = re.match(r"k_ns_fused<(\d+x\d+),(true|false)>", n)
+    if m:
+        return f"k_ns_fused<{m.group(1)},{'bwd' if m.group(2) == 'true' else 'fwd'}>"
+    m = re.match(r"k_row_gemm_dma<(\d+x\d+),(\d+),(\d+),(true|false)>", n)
+    if m:
+        epi = {"0": "store", "1": "axpby", "2": "axpby_dual"}[m.group(3)]
+        return f"k_row_gemm_dma<{m.group(1)},{m.group(2)},{epi},{'Bks' if m.group(4) == 'true' else 'Bkc'}>"
+    m = re.match(r"(k_token_reduce(?:_rows)?_dma)<(\d+x\d+)>", n)
+    if m:
+        return f"{m.group(1)}<{m.group(2)}>"
+    return n.split("<")[0]
+
+
+def load_traffic(cfg):
+    """HBM bytes per launch of every kernel and per step, read from the committed counter summary of this
+    configuration (FETCH_SIZE / WRITE_SIZE of two `rocprofv3 --pmc` runs, already scaled by the copy calibration
+    the file states).  Returns ({library label: bytes per launch}, bytes per step or None); empty when the file is
+    missing or a line does not parse -- the bench line then carries `traffic: null`."""
+    import re
+    per_kernel, per_step = {}, None
+    try:
+        with open(TRAFFIC_PROFILE.format(cfg=cfg)) as f:
+            for line in f:
+                m = re.match(r"^(.*\S)\s+(\d+)\s+([0-9.]+)\s+([0-9.]+)\s*$", line)
+                if m and "k_" in m.group(1):
+                    per_kernel[_library_label(m.group(1))] = (float(m.group(3)) + float(m.group(4))) * 2 ** 20
+                m = re.match(r"^per step.*read\s+([0-9.]+) MiB, write\s+([0-9.]+) MiB", line)
+                if m:
+                    per_step = (float(m.group(1)) + float(m.group(2))) * 2 ** 20
+    except OSError:
+        pass
+    return per_kernel, per_step
 
 
 def algorithmic_flops(b, L, d, dh, C, ns_steps=5):
@@ -80,6 +105,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (three times): the known-size kernel that scales the "
                          "FETCH_SIZE / WRITE_SIZE counters of a `rocprofv3 --pmc` run of this command")
+    ap.add_argument("--mfma-calibration", action="store_true",
+                    help="also run the library's pure matrix-instruction kernel (three times, 1024 workgroups): the kernel "
+                         "of known matrix-pipe occupancy that scales a matrix-busy counter of a `rocprofv3 --pmc` run")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures the one-GPU operation only: heads (b = B*H) are independent, so N GPUs would each run "
@@ -127,6 +155,14 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    if args.mfma_calibration:
+        buf = torch.empty(1024 * 256, dtype=torch.float32, device="cuda:0")
+        for _ in range(3):
+            _lib.check(_lib.lib().lact_mfma_calibration(1024, 4000, ctypes.c_void_p(buf.data_ptr()),
+                                                        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+        torch.cuda.synchronize()
+        del buf
+
     if args.no_overlap:
         _lib.lib().lact_set_option(_lib.OPT_STREAM_OVERLAP, 0)
     for _ in range(args.warmup):
@@ -154,6 +190,7 @@ def main():
         "op_tflops": op_tflops, "op_frac_of_bf16_peak": op_tflops / PEAK_BF16_TFLOPS,
     }
 
+    traffic, step_traffic = load_traffic(args.config)
     # ---- per-kernel durations: the same K steps again with HIP events around every launch, on the stream
     #      the kernels run on (a second pass, so that the events do not perturb `value`)
     if not args.no_kernel_profile:
@@ -177,8 +214,7 @@ def main():
         achieved = dom["flops"] / dom["launches"] / (avg_ms * 1e-3) / 1e12
         res["roofline"] = {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                            "frac": achieved / PEAK_BF16_TFLOPS,
-                           "traffic": (MEASURED_TRAFFIC_MIB[dom_name] * 2 ** 20
-                                       if args.config == "c1" and dom_name in MEASURED_TRAFFIC_MIB else None),
+                           "traffic": traffic.get(dom_name),
                            "kernel": dom_name,
                            "avg_launch_ms": avg_ms, "launches_per_step": dom["launches"] / args.steps,
                            "share_of_kernel_time": dom["ms"] / total_ms}
@@ -188,11 +224,11 @@ def main():
               "tflops": (r["flops"] / (r["ms"] * 1e-3) / 1e12) if r["ms"] > 0 and r["flops"] > 0 else None}
              for r in rows], key=lambda r: -r["ms_per_step"])
         res["kernel_ms_per_step"] = total_ms / args.steps
-    if args.config == "c1":
-        gbps = MEASURED_STEP_TRAFFIC_MIB * 2 ** 20 / (ms_per_step * 1e-3) / 1e9
-        res["step_hbm"] = {"bytes_per_step": MEASURED_STEP_TRAFFIC_MIB * 2 ** 20, "achieved": gbps, "peak": PEAK_HBM_GBPS,
+    if step_traffic:
+        gbps = step_traffic / (ms_per_step * 1e-3) / 1e9
+        res["step_hbm"] = {"bytes_per_step": step_traffic, "achieved": gbps, "peak": PEAK_HBM_GBPS,
                            "unit": "GB/s", "frac": gbps / PEAK_HBM_GBPS,
-                           "source": "profiles/c1_fwd_bwd_hbm_traffic_pmc.txt (FETCH_SIZE + WRITE_SIZE of every kernel of a step)"}
+                           "source": f"profiles/{args.config}_fwd_bwd_hbm_traffic_pmc.txt (FETCH_SIZE + WRITE_SIZE of every kernel of a step)"}
 
     # ---- CPU baseline: the oracle (a restatement of the reference's non-fused PyTorch op) on the host cores
     if not args.no_cpu_baseline:

@@ -207,6 +207,10 @@ int lact_check_async_error(void);
  * the device, writes a JSON array of {kernel, site, launches, ms, flops} into buf and resets the
  * records.  Not thread-safe; meant for benchmarking. */
 int lact_profile_enable(int on);
+/* Calibration kernel for matrix-pipe counters (`rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES ...`): `blocks` workgroups of
+ * four waves that issue nothing but bf16 matrix instructions, `iters` x 8 each; out: blocks * 256 floats.  What the
+ * counter reads for it is the reading of a fully busy matrix pipe.  No counterpart in the reference. */
+int lact_mfma_calibration(int32_t blocks, int32_t iters, float* out, void* stream);
 int lact_profile_report(char* buf, size_t cap);
 
 #ifdef __cplusplus

@@ -38,7 +38,7 @@ OPT_STREAM_OVERLAP, OPT_FUSED_NEWTON_SCHULZ, OPT_NS_BARRIER_SPIN_LIMIT = 0, 1, 2
 EXPORTS = ("lact_last_error", "lact_version", "lact_query_sizes", "lact_forward", "lact_forward_from_state", "lact_backward",
            "lact_newton_schulz_workspace_bytes", "lact_newton_schulz", "lact_newton_schulz_static_capacity",
            "lact_newton_schulz_static", "lact_newton_schulz_backward_workspace_bytes", "lact_newton_schulz_backward",
-           "lact_check_async_error", "lact_set_option", "lact_profile_enable",
+           "lact_check_async_error", "lact_mfma_calibration", "lact_set_option", "lact_profile_enable",
            "lact_profile_report", "lact_layer_pre_forward", "lact_layer_pre_backward", "lact_layer_lr_forward",
            "lact_layer_lr_backward", "lact_layer_post_forward", "lact_layer_post_dw_rows", "lact_layer_post_backward")
 
@@ -77,6 +77,8 @@ def lib():
     L.lact_newton_schulz_backward_workspace_bytes.restype = c_size_t
     L.lact_newton_schulz_backward.argtypes = [c_int32, c_int32, c_int32, vp, vp, vp, c_int32, POINTER(c_float), c_int32, vp, vp]
     L.lact_newton_schulz_backward.restype = c_int32
+    L.lact_mfma_calibration.argtypes = [c_int32, c_int32, vp, vp]
+    L.lact_mfma_calibration.restype = c_int32
     L.lact_check_async_error.argtypes = []
     L.lact_check_async_error.restype = c_int32
     L.lact_set_option.argtypes = [c_int32, c_int32]

@@ -894,8 +894,21 @@ struct Runner {
       T* kl0 = scr<T>(P.t_kl[0]);
       T* kl2 = scr<T>(P.t_kl[1]);
       const long long klbs = (long long)P.Tcap * d.d;
-      LACT_LAUNCH("k_lr_scale_rows", "update_lr_k", 0.0, (k_lr_scale_rows<T>), dim3((unsigned)(((long long)T_ * d.d / 4 + 255) / 256), d.b), dim3(256), s,
-                  kc, d.k_ld, d.k_bs, lr0 + st.start, lr2 + st.start, (long long)d.kv_len, T_, d.d, kl0, kl2, klbs);
+      // k * lr0, k * lr2 depend on the inputs only and are first read by the token reduction: they are written on the
+      // tail stream beside the hidden stage (after everything enqueued so far, which includes the previous update's
+      // reduction that read the same two buffers)
+      hipEvent_t kl_ready = nullptr;
+      {
+        const bool aside = s_tail != s_main && side;
+        if (aside) { wait_for(s_tail, s_main); s = s_tail; }
+        LACT_LAUNCH("k_lr_scale_rows", "update_lr_k", 0.0, (k_lr_scale_rows<T>), dim3((unsigned)(((long long)T_ * d.d / 4 + 255) / 256), d.b), dim3(256), s,
+                    kc, d.k_ld, d.k_bs, lr0 + st.start, lr2 + st.start, (long long)d.kv_len, T_, d.d, kl0, kl2, klbs);
+        if (aside) {
+          kl_ready = side->event();
+          (void)hipEventRecord(kl_ready, s_tail);
+          s = s_main;
+        }
+      }
       {
         HiddenParams hp = hidden_params(T_, kc, d.k_ld, d.k_bs, vc, d.v_ld, d.v_bs, ver);
         hp.lr0 = lr0 + st.start; hp.lr1 = lr1 + st.start; hp.lr2 = lr2 + st.start; hp.bslr = d.kv_len;
@@ -916,6 +929,7 @@ struct Runner {
       // what enters the weights (the next update and its backward would read it; the caller gets its own copy)
       const bool d_unread = P.muon && !d.muon_replaces_weight && u + 1 == P.nupd;
       int dw_slots = 0;
+      if (kl_ready) (void)hipStreamWaitEvent(s_main, kl_ready, 0);
       {
         TokenReduceJob jobs[3];
         memset(jobs, 0, sizeof(jobs));
@@ -1924,6 +1938,31 @@ int lact_check_async_error(void) {
           "the results of those steps are NaN (compute units held by another process or kernel; raise "
           "LACT_OPT_NS_BARRIER_SPIN_LIMIT or switch LACT_OPT_FUSED_NEWTON_SCHULZ off)";
   return (int)std::min<unsigned>(n, 0x7fffffffu);
+}
+
+// Back-to-back matrix instructions on every SIMD of every compute unit: the kernel of known matrix-pipe occupancy
+// (all of it) that scales a matrix-busy counter of `rocprofv3 --pmc`, as a plain copy scales the byte counters.
+__global__ __launch_bounds__(256) void k_mfma_calibration(int iters, float* out) {
+  f32x16 acc[8];
+  for (int i = 0; i < 8; ++i)
+    for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
+  bf16x8 a, b;
+  for (int j = 0; j < 8; ++j) { a[j] = (__bf16)(float)((threadIdx.x + j) & 7); b[j] = (__bf16)(float)((threadIdx.x * 3 + j) & 3); }
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[i], 0, 0, 0);
+  }
+  float sum = 0.f;
+  for (int i = 0; i < 8; ++i)
+    for (int j = 0; j < 16; ++j) sum += acc[i][j];
+  out[(size_t)blockIdx.x * 256 + threadIdx.x] = sum;
+}
+
+int lact_mfma_calibration(int32_t blocks, int32_t iters, float* out, void* stream) {
+  if (blocks <= 0 || iters <= 0 || !out) return fail("lact_mfma_calibration: bad arguments");
+  hipLaunchKernelGGL(k_mfma_calibration, dim3(blocks), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), iters, out);
+  LACT_CHECK_LAUNCH();
+  return 0;
 }
 
 int lact_profile_enable(int on) {
