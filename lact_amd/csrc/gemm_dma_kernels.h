@@ -25,6 +25,111 @@ struct RowGemmDmaParams {
   TileMap map;        // tiles of M, tiles of N, batch
 };
 
+// The phases of one output tile (rows from m0, columns from n0) of batch entry z: one per term.
+// B_KS: the B operands are [K, N] (N contiguous) instead of [N, K].
+template <class TS, int NT, bool B_KS>
+__device__ __forceinline__ void row_gemm_phases(const RowGemmParams<NT>& p, int m0, int n0, int z, DmaPhase<1> (&ph)[NT]) {
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    ph[t].a.base = reinterpret_cast<const uint16_t*>(p.t[t].A) + z * p.t[t].bsA + (size_t)m0 * p.t[t].lda;
+    ph[t].a.ld = p.t[t].lda; ph[t].a.rows = p.M - m0; ph[t].a.ks = 0;
+    ph[t].b[0].base = reinterpret_cast<const uint16_t*>(p.t[t].B) + z * p.t[t].bsB + (B_KS ? (size_t)n0 : (size_t)n0 * p.t[t].ldb);
+    ph[t].b[0].ld = p.t[t].ldb; ph[t].b[0].rows = p.N - n0; ph[t].b[0].ks = B_KS;
+    ph[t].nb = 1;
+    ph[t].K = p.t[t].K;
+  }
+}
+
+// EPI_STORE / EPI_AXPBY: the tile staged in LDS as bf16 (StageTile<TS, 2>, = round(acc)) goes out in whole rows; all
+// threads of the block take part.
+template <class TS, int NT, int EPI>
+__device__ __forceinline__ void row_gemm_copy_out_b16(const RowGemmParams<NT>& p, int m0, int n0, int z, const char* smem) {
+  using ST = StageTile<TS, 2>;
+  const int r0 = ST::row0(), c0 = ST::col0();
+  if (ST::active() && n0 + c0 < p.N) {
+    const char* src = smem + (r0 * ST::LD + c0) * 2;
+    uint16_t* dst = reinterpret_cast<uint16_t*>(p.out) + z * p.bso + (size_t)(m0 + r0) * p.ldo + n0 + c0;
+    const uint16_t* aux = reinterpret_cast<const uint16_t*>(p.aux) + z * p.bsaux + (size_t)(m0 + r0) * p.ldaux + n0 + c0;
+    const size_t dstep = (size_t)ST::RPP * p.ldo, astep = (size_t)ST::RPP * p.ldaux;
+    const bool blend = EPI == EPI_AXPBY || p.accumulate;
+    // all auxiliary loads first (no store in between may alias them), then blend and store
+    uint4 w[ST::PASSES];
+    if (blend) {
+      const uint16_t* ap = EPI == EPI_STORE ? dst : aux;
+      const size_t st = EPI == EPI_STORE ? dstep : astep;
+#pragma unroll
+      for (int ps = 0; ps < ST::PASSES; ++ps) {
+        const int r = r0 + ps * ST::RPP;
+        w[ps] = (r < TS::BM && m0 + r < p.M) ? *reinterpret_cast<const uint4*>(ap + ps * st) : make_uint4(0, 0, 0, 0);
+      }
+    }
+    const float al = EPI == EPI_STORE ? 1.f : p.alpha, be = EPI == EPI_STORE ? 1.f : p.beta;
+    uint16_t* dst2 = (EPI == EPI_STORE && p.out2) ? reinterpret_cast<uint16_t*>(p.out2) + (dst - reinterpret_cast<uint16_t*>(p.out)) : nullptr;
+    // LDS reads in unconditional groups of 8 (a branch per row would put every read's latency in line)
+    uint4 ug[8];
+#pragma unroll
+    for (int ps = 0; ps < ST::PASSES; ++ps) {
+      if (ps % 8 == 0) {
+#pragma unroll
+        for (int g = 0; g < 8; ++g)
+          if (ps + g < ST::PASSES) ug[g] = ST::read16(src, r0, ps + g);
+      }
+      const int r = r0 + ps * ST::RPP;
+      if (r < TS::BM && m0 + r < p.M) {
+        uint4 u = ug[ps % 8];
+        if (blend) {
+          // the staged values are round(acc); each product and the sum are tensors of their own in the reference
+          uint32_t uu[4] = {u.x, u.y, u.z, u.w}, ww[4] = {w[ps].x, w[ps].y, w[ps].z, w[ps].w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float lo = round_bf16(al * __uint_as_float(uu[j] << 16)) + round_bf16(be * __uint_as_float(ww[j] << 16));
+            const float hi = round_bf16(al * __uint_as_float(uu[j] & 0xffff0000u)) + round_bf16(be * __uint_as_float(ww[j] & 0xffff0000u));
+            uu[j] = (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+          }
+          u = make_uint4(uu[0], uu[1], uu[2], uu[3]);
+        }
+        *reinterpret_cast<uint4*>(dst) = u;
+        if (dst2) {
+          uint32_t uu[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            uu[j] = (uint32_t)f32_to_bf16(p.alpha2 * __uint_as_float(uu[j] << 16)) |
+                    ((uint32_t)f32_to_bf16(p.alpha2 * __uint_as_float(uu[j] & 0xffff0000u)) << 16);
+          *reinterpret_cast<uint4*>(dst2) = make_uint4(uu[0], uu[1], uu[2], uu[3]);
+        }
+      }
+      dst += dstep;
+      if (dst2) dst2 += dstep;
+    }
+  }
+}
+
+// Transposed copies of the fp32 tile staged in LDS (StageTile<TS, 4>): lanes run along n (conflict-free LDS reads),
+// each lane owns 8 consecutive m.  All threads of the block take part.
+template <class TS, int NT>
+__device__ __forceinline__ void row_gemm_copy_out_transposed(const RowGemmParams<NT>& p, uint16_t* out_ct, bool tr, int m0, int n0, int z, const char* smem) {
+  using ST = StageTile<TS, 4>;
+  const float* tile = reinterpret_cast<const float*>(smem);
+#pragma unroll 2
+  for (int id = threadIdx.x; id < TS::BN * (TS::BM / 8); id += DMA_THREADS) {
+    const int nl = id % TS::BN, ml = (id / TS::BN) * 8;
+    const int m = m0 + ml, n = n0 + nl;
+    if (m >= p.M || n >= p.N) continue;
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = tile[(ml + j) * ST::LD + nl];
+    const size_t off = z * p.bso + (size_t)n * p.M + m;
+    if (p.out_t && tr) {
+      Elem<float>::store4(p.out_t + off, v[0], v[1], v[2], v[3]);
+      Elem<float>::store4(p.out_t + off + 4, v[4], v[5], v[6], v[7]);
+    }
+    if (out_ct) {
+      Elem<uint16_t>::store4(out_ct + off, v[0], v[1], v[2], v[3]);
+      Elem<uint16_t>::store4(out_ct + off + 4, v[4], v[5], v[6], v[7]);
+    }
+  }
+}
+
 // One output tile (bx, by) of batch entry z.  B_KS: the B operands are [K, N] (N contiguous) instead of [N, K].
 // SC1: the operands were written by other compute units during this kernel (loads bypass the vector L1); the
 // auxiliary tile of the blending epilogues is always one this block wrote itself or an earlier kernel wrote.
@@ -37,17 +142,8 @@ __device__ __forceinline__ void row_gemm_tile(const RowGemmDmaParams<NT>& pp, in
   const RowGemmParams<NT>& p = pp.g;
   const int m0 = bx * TS::BM, n0 = by * TS::BN;
   DmaPhase<1> ph[NT];
-#pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    ph[t].a.base = reinterpret_cast<const uint16_t*>(p.t[t].A) + z * p.t[t].bsA + (size_t)m0 * p.t[t].lda;
-    ph[t].a.ld = p.t[t].lda; ph[t].a.rows = p.M - m0; ph[t].a.ks = 0;
-    ph[t].b[0].base = reinterpret_cast<const uint16_t*>(p.t[t].B) + z * p.t[t].bsB + (B_KS ? (size_t)n0 : (size_t)n0 * p.t[t].ldb);
-    ph[t].b[0].ld = p.t[t].ldb; ph[t].b[0].rows = p.N - n0; ph[t].b[0].ks = B_KS;
-    ph[t].nb = 1;
-    ph[t].K = p.t[t].K;
-  }
-  f32x16 acc[1][TS::TM][TS::TN];
-  zero_acc<TS>(acc[0]);
+  row_gemm_phases<TS, NT, B_KS>(p, m0, n0, z, ph);
+  f32x16 acc[1][TS::TM][TS::TN];   // defined on the matrix waves' path only: the loader waves' registers stay free for their copies
   LACT_TS(0);
   Pipe pipe(smem, ph);
   const bool loader = Pipe::is_loader();
@@ -55,6 +151,7 @@ __device__ __forceinline__ void row_gemm_tile(const RowGemmDmaParams<NT>& pp, in
   if (loader) {
     pipe.template load_all<Pipe::loads(1)>();
   } else {
+    zero_acc<TS>(acc[0]);
     int step = 0;
 #pragma unroll
     for (int t = 0; t < NT; ++t) pipe.template run_phase<1, false, B_KS>(p.t[t].K / DMA_BK, step, acc);
@@ -70,63 +167,7 @@ __device__ __forceinline__ void row_gemm_tile(const RowGemmDmaParams<NT>& pp, in
       LACT_FOR_QUADS(TS) ST::put4(lb, tm, tn, g, acc[0][tm][tn][4 * g], acc[0][tm][tn][4 * g + 1], acc[0][tm][tn][4 * g + 2], acc[0][tm][tn][4 * g + 3]);
     }
     __syncthreads();
-    const int r0 = ST::row0(), c0 = ST::col0();
-    if (ST::active() && n0 + c0 < p.N) {
-      const char* src = smem + (r0 * ST::LD + c0) * 2;
-      uint16_t* dst = reinterpret_cast<uint16_t*>(p.out) + z * p.bso + (size_t)(m0 + r0) * p.ldo + n0 + c0;
-      const uint16_t* aux = reinterpret_cast<const uint16_t*>(p.aux) + z * p.bsaux + (size_t)(m0 + r0) * p.ldaux + n0 + c0;
-      const size_t dstep = (size_t)ST::RPP * p.ldo, astep = (size_t)ST::RPP * p.ldaux;
-      const bool blend = EPI == EPI_AXPBY || p.accumulate;
-      // all auxiliary loads first (no store in between may alias them), then blend and store
-      uint4 w[ST::PASSES];
-      if (blend) {
-        const uint16_t* ap = EPI == EPI_STORE ? dst : aux;
-        const size_t st = EPI == EPI_STORE ? dstep : astep;
-#pragma unroll
-        for (int ps = 0; ps < ST::PASSES; ++ps) {
-          const int r = r0 + ps * ST::RPP;
-          w[ps] = (r < TS::BM && m0 + r < p.M) ? *reinterpret_cast<const uint4*>(ap + ps * st) : make_uint4(0, 0, 0, 0);
-        }
-      }
-      const float al = EPI == EPI_STORE ? 1.f : p.alpha, be = EPI == EPI_STORE ? 1.f : p.beta;
-      uint16_t* dst2 = (EPI == EPI_STORE && p.out2) ? reinterpret_cast<uint16_t*>(p.out2) + (dst - reinterpret_cast<uint16_t*>(p.out)) : nullptr;
-      // LDS reads in unconditional groups of 8 (a branch per row would put every read's latency in line)
-      uint4 ug[8];
-#pragma unroll
-      for (int ps = 0; ps < ST::PASSES; ++ps) {
-        if (ps % 8 == 0) {
-#pragma unroll
-          for (int g = 0; g < 8; ++g)
-            if (ps + g < ST::PASSES) ug[g] = ST::read16(src, r0, ps + g);
-        }
-        const int r = r0 + ps * ST::RPP;
-        if (r < TS::BM && m0 + r < p.M) {
-          uint4 u = ug[ps % 8];
-          if (blend) {
-            // the staged values are round(acc); each product and the sum are tensors of their own in the reference
-            uint32_t uu[4] = {u.x, u.y, u.z, u.w}, ww[4] = {w[ps].x, w[ps].y, w[ps].z, w[ps].w};
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              const float lo = round_bf16(al * __uint_as_float(uu[j] << 16)) + round_bf16(be * __uint_as_float(ww[j] << 16));
-              const float hi = round_bf16(al * __uint_as_float(uu[j] & 0xffff0000u)) + round_bf16(be * __uint_as_float(ww[j] & 0xffff0000u));
-              uu[j] = (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
-            }
-            u = make_uint4(uu[0], uu[1], uu[2], uu[3]);
-          }
-          *reinterpret_cast<uint4*>(dst) = u;
-          if (dst2) {
-            uint32_t uu[4] = {u.x, u.y, u.z, u.w};
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-              uu[j] = (uint32_t)f32_to_bf16(p.alpha2 * __uint_as_float(uu[j] << 16)) |
-                      ((uint32_t)f32_to_bf16(p.alpha2 * __uint_as_float(uu[j] & 0xffff0000u)) << 16);
-            *reinterpret_cast<uint4*>(dst2) = make_uint4(uu[0], uu[1], uu[2], uu[3]);
-          }
-        }
-        dst += dstep;
-        if (dst2) dst2 += dstep;
-      }
-    }
+    row_gemm_copy_out_b16<TS, NT, EPI>(p, m0, n0, z, smem);
   } else {
     using ST = StageTile<TS, 4>;
     char* lb = smem + ST::lane_base();
@@ -148,7 +189,7 @@ __device__ __forceinline__ void row_gemm_tile(const RowGemmDmaParams<NT>& pp, in
         const int r = r0 + ps * ST::RPP;
         x4[ps] = (r < TS::BM && m0 + r < p.M) ? *reinterpret_cast<const float4*>(aux + ps * astep) : make_float4(0.f, 0.f, 0.f, 0.f);
       }
-        uint4 ag[8];
+      uint4 ag[8];
 #pragma unroll
       for (int ps = 0; ps < ST::PASSES; ++ps) {
         if (ps % 8 == 0) {
@@ -175,29 +216,7 @@ __device__ __forceinline__ void row_gemm_tile(const RowGemmDmaParams<NT>& pp, in
     }
     if (need_t) {
       __syncthreads();
-      // transposed copies: lanes run along n (conflict-free LDS reads), each lane owns 8 consecutive m
-      const float* tile = reinterpret_cast<const float*>(smem);
-      constexpr int TP = TS::BN * (TS::BM / 8) / TS::THREADS;
-      static_assert(TS::THREADS % TS::BN == 0 || TS::BN % TS::THREADS == 0 || TS::BN == 192, "transposed pass mapping");
-#pragma unroll 2
-      for (int id = threadIdx.x; id < TS::BN * (TS::BM / 8); id += DMA_THREADS) {
-        const int nl = id % TS::BN, ml = (id / TS::BN) * 8;
-        const int m = m0 + ml, n = n0 + nl;
-        if (m >= p.M || n >= p.N) continue;
-        float v[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = tile[(ml + j) * ST::LD + nl];
-        const size_t off = z * p.bso + (size_t)n * p.M + m;
-        if (p.out_t && tr) {
-          Elem<float>::store4(p.out_t + off, v[0], v[1], v[2], v[3]);
-          Elem<float>::store4(p.out_t + off + 4, v[4], v[5], v[6], v[7]);
-        }
-        if (pp.out_ct) {
-          Elem<uint16_t>::store4(pp.out_ct + off, v[0], v[1], v[2], v[3]);
-          Elem<uint16_t>::store4(pp.out_ct + off + 4, v[4], v[5], v[6], v[7]);
-        }
-      }
-      (void)TP;
+      row_gemm_copy_out_transposed<TS, NT>(p, pp.out_ct, tr, m0, n0, z, smem);
     }
   }
   LACT_TS(3);
@@ -264,8 +283,6 @@ __global__ __launch_bounds__(DMA_THREADS) void k_apply_hidden_dma(const HiddenDm
   ph[0].K = p.d;
   const int nk = (p.d + DMA_BK - 1) / DMA_BK;
   f32x16 acc[2][TS::TM][TS::TN];
-  zero_acc<TS>(acc[0]);
-  zero_acc<TS>(acc[1]);
   LACT_TS(0);
   Pipe pipe(smem, ph);
   const bool loader = Pipe::is_loader();
@@ -273,6 +290,8 @@ __global__ __launch_bounds__(DMA_THREADS) void k_apply_hidden_dma(const HiddenDm
   if (loader) {
     pipe.template load_all<Pipe::loads(2)>();
   } else {
+    zero_acc<TS>(acc[0]);
+    zero_acc<TS>(acc[1]);
     int step = 0;
     pipe.template run_phase<2>(nk, step, acc);
   }
@@ -315,13 +334,13 @@ __device__ __forceinline__ void three_acc_mainloop(const HiddenDmaParams& pp, ch
   ph[1].nb = 1;
   ph[1].K = p.d;
   const int nk = (p.d + DMA_BK - 1) / DMA_BK;
-  zero_acc<TS>(a02[0]);
-  zero_acc<TS>(a02[1]);
-  zero_acc<TS>(a1[0]);
   Pipe pipe(smem, ph);
   if (Pipe::is_loader()) {
     pipe.template load_all<Pipe::loads(1)>();
   } else {
+    zero_acc<TS>(a02[0]);
+    zero_acc<TS>(a02[1]);
+    zero_acc<TS>(a1[0]);
     int step = 0;
     pipe.template run_phase<2>(nk, step, a02);
     pipe.template run_phase<1, false, true>(nk, step, a1);
@@ -461,12 +480,12 @@ __global__ __launch_bounds__(DMA_THREADS) void k_update_bwd_hidden_dma(const Hid
   ph[0].nb = ph[1].nb = ph[2].nb = 2;
   const int nk = (p.d + DMA_BK - 1) / DMA_BK;
   f32x16 aw[2][TS::TM][TS::TN], ag[2][TS::TM][TS::TN], ay[2][TS::TM][TS::TN];
-  zero_acc<TS>(aw[0]); zero_acc<TS>(aw[1]); zero_acc<TS>(ag[0]); zero_acc<TS>(ag[1]); zero_acc<TS>(ay[0]); zero_acc<TS>(ay[1]);
   Pipe pipe(smem, ph);
   const bool loader = Pipe::is_loader();
   if (loader) {
     pipe.template load_all<Pipe::loads(2)>();
   } else {
+    zero_acc<TS>(aw[0]); zero_acc<TS>(aw[1]); zero_acc<TS>(ag[0]); zero_acc<TS>(ag[1]); zero_acc<TS>(ay[0]); zero_acc<TS>(ay[1]);
     int step = 0;
     pipe.template run_phase<2>(nk, step, aw);
     pipe.template run_phase<2>(nk, step, ag);
@@ -566,15 +585,15 @@ __global__ __launch_bounds__(DMA_THREADS) void k_update_bwd_hidden_kept_dma(cons
   ph[2].nb = 2;
   ph[2].K = halves * 64;
   f32x16 ag[2][TS::TM][TS::TN], ay[1][TS::TM][TS::TN];
-  zero_acc<TS>(ag[0]);
-  zero_acc<TS>(ag[1]);
-  zero_acc<TS>(ay[0]);
   LACT_TS(0);
   Pipe pipe(smem, ph);
   const bool loader = Pipe::is_loader();
   if (loader) {
     pipe.template load_all<Pipe::loads(1)>();
   } else {
+    zero_acc<TS>(ag[0]);
+    zero_acc<TS>(ag[1]);
+    zero_acc<TS>(ay[0]);
     int step = 0;
     pipe.template run_phase<1, false, true>(nk, step, ay);
     pipe.template run_phase<2>(nk, step, ag);
@@ -703,12 +722,12 @@ __device__ __forceinline__ void token_reduce_dma_block(const TokenReduceDmaParam
     ph[t].a.ktail = ph[t].b[0].ktail = klen % DMA_BK;
   }
   f32x16 acc[1][TS::TM][TS::TN];
-  zero_acc<TS>(acc[0]);
   Pipe pipe(smem, ph);
   const bool loader = Pipe::is_loader();
   if (loader) {
     pipe.template load_all<Pipe::loads(1)>();
   } else {
+    zero_acc<TS>(acc[0]);
     int step = 0;
     pipe.template run_phase<1, true, true>(ph[0].K / DMA_BK, step, acc);
     pipe.template run_phase<1, true, true>(ph[1].K / DMA_BK, step, acc);
