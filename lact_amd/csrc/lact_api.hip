@@ -821,6 +821,12 @@ struct Runner {
               const float* lr1, const float* lr2, const float* mom, T* out, float* const w_out[3], float* const m_out[3],
               const float* const m_in[3]) {
     const dim3 rowgrid(ceil_div(P.g.maxrows(), 4), 3 * d.b);
+    // what depends on the inputs only may start on the tail stream right here, beside the first kernels of the call
+    hipEvent_t entry = nullptr;
+    if (s_tail != s_main && side) {
+      entry = side->event();
+      (void)hipEventRecord(entry, s_main);
+    }
     // carried momentum state: packed like every other state array (a device-to-device copy node when captured)
     if (P.state_in && P.nupd > 0)
       for (int j = 0; j < 3; ++j)
@@ -895,12 +901,16 @@ struct Runner {
       T* kl2 = scr<T>(P.t_kl[1]);
       const long long klbs = (long long)P.Tcap * d.d;
       // k * lr0, k * lr2 depend on the inputs only and are first read by the token reduction: they are written on the
-      // tail stream beside the hidden stage (after everything enqueued so far, which includes the previous update's
-      // reduction that read the same two buffers)
+      // tail stream beside the hidden stage -- after everything enqueued so far (which includes the previous update's
+      // reduction that read the same two buffers), the first update's already beside the state set-up of the call
       hipEvent_t kl_ready = nullptr;
       {
         const bool aside = s_tail != s_main && side;
-        if (aside) { wait_for(s_tail, s_main); s = s_tail; }
+        if (aside) {
+          if (u == 0 && entry) (void)hipStreamWaitEvent(s_tail, entry, 0);
+          else wait_for(s_tail, s_main);
+          s = s_tail;
+        }
         LACT_LAUNCH("k_lr_scale_rows", "update_lr_k", 0.0, (k_lr_scale_rows<T>), dim3((unsigned)(((long long)T_ * d.d / 4 + 255) / 256), d.b), dim3(256), s,
                     kc, d.k_ld, d.k_bs, lr0 + st.start, lr2 + st.start, (long long)d.kv_len, T_, d.d, kl0, kl2, klbs);
         if (aside) {
