@@ -122,8 +122,26 @@ struct SideCtx {
   hipStream_t tail = nullptr;        // second side stream: results of the update chain that nothing in the call waits for
   std::vector<hipEvent_t> ev;
   size_t next = 0;
-  hipEvent_t fused_done = nullptr;   // completion of the newest fused Newton-Schulz kernel of this process
-  bool fused_recorded = false;
+  // Fused Newton-Schulz kernels of this process must not overlap each other (each needs its groups resident as a whole).
+  // Launches on one stream follow each other anyway; an event is recorded (on the stream of the newest launch, at the
+  // time the next launch arrives) only when that next launch comes from another stream -- a record behind every launch
+  // would put ~3 us between the kernel and whatever follows it on the caller's stream.
+  hipEvent_t fused_done = nullptr;
+  hipStream_t fused_stream = nullptr;
+  bool fused_any = false;
+  void order_fused_launch(hipStream_t s) {
+    if (fused_any && fused_stream != s) {
+      if (!fused_done) (void)hipEventCreateWithFlags(&fused_done, hipEventDisableTiming);
+      if (hipEventRecord(fused_done, fused_stream) == hipSuccess) {
+        (void)hipStreamWaitEvent(s, fused_done, 0);
+      } else {   // that stream no longer exists: whatever it still runs is waited for the hard way
+        (void)hipGetLastError();
+        (void)hipDeviceSynchronize();
+      }
+    }
+    fused_stream = s;
+    fused_any = true;
+  }
   int cus = 0;                       // compute units of the device (0: not asked yet)
   unsigned* sticky = nullptr;        // device address of this device's count of barrier time-outs
   hipEvent_t event() {
@@ -575,13 +593,9 @@ struct Runner {
     for (int z0 = 0; z0 < B.n; z0 += per) {
       p.z0 = z0; p.n = std::min(per, B.n - z0); p.sync = sync + (size_t)z0 * 32;
       const int grid = 8 * ((p.n + 7) / 8) * nbm;
-      // fused launches of this process never overlap each other (each needs its groups resident as a whole)
-      if (side->fused_recorded) (void)hipStreamWaitEvent(s, side->fused_done, 0);
+      side->order_fused_launch(s);
       LACT_LAUNCH_SMEM(name.c_str(), BWD ? "ns_bwd" : "ns_fwd", terms * 2.0 * B.r * B.r * B.c * P.S * p.n,
                        (k_ns_fused<TS, BWD>), dim3(grid), dim3(DMA_THREADS), SM, s, p);
-      if (!side->fused_done) (void)hipEventCreateWithFlags(&side->fused_done, hipEventDisableTiming);
-      (void)hipEventRecord(side->fused_done, s);
-      side->fused_recorded = true;
     }
   }
   template <bool BWD>
