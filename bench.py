@@ -1,6 +1,6 @@
 """Benchmark of the TTT operation on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1|c2|c4] [--no-cpu-baseline]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1|c2|c3|c4|layer] [--no-cpu-baseline]
 
 One step = forward + backward of block_causal_lact_swiglu over one batch of seeded synthetic input
 that is resident in HBM before the timed region.  Prints one JSON line (metric: tokens/s, tokens = B*L).
@@ -32,6 +32,11 @@ CONFIGS = {
     "c3": (1, 6, 9216, 128, 256, 8192, 1003,
            "config 3: fast_weight_swish_glu_weight_norm_mini_batch_apply forward only, NVS shape b=6, d=128, dh=256, "
            "update on 8192 tokens then apply on 1024, Muon with 5 classic Newton-Schulz steps"),
+    # the layer around the operation (not a BASELINE configuration: the callers either side of the path, measured)
+    "layer": (4, 4, 4096, 384, 384, 2048, 1005,
+              "layer: CausalLaCTSwiGLUWithSlidingWindowAttn fwd+bwd under bf16 autocast, 760M shape (dim 1536 = 4 heads of "
+              "384, 12 attention heads of 128, window 2048), B=4, L=4096, chunk 2048, Muon + momentum; projections are "
+              "rocBLAS GEMMs through torch.nn.Linear, attention is torch's blocked SDPA, the rest is this library"),
 }
 
 
@@ -147,6 +152,29 @@ def main():
             with torch.no_grad():
                 return nvs.fast_weight_swish_glu_weight_norm_mini_batch_apply(*dev3, program, 5)[0]
 
+    if args.config == "layer":
+        from lact_amd import layers
+        torch.manual_seed(seed)
+        layer = layers.CausalLaCTSwiGLUWithSlidingWindowAttn(dim=H * d, head_dim=d, attn_head_dim=128, lact_chunk_size=C,
+                                                             window_size=2048).to("cuda:0")
+        xin = torch.randn(B, L, H * d, generator=torch.Generator().manual_seed(seed)).to("cuda:0").requires_grad_(True)
+        gout = torch.randn(B, L, H * d, generator=torch.Generator().manual_seed(seed + 1)).bfloat16().to("cuda:0")
+        no_attention = [False]
+        real_attention = layers.sliding_window_attention
+
+        def attention_or_nothing(q_, k_, v_, window):   # the TTT branch alone: attention replaced by its value input
+            return v_ if no_attention[0] else real_attention(q_, k_, v_, window)
+        layers.sliding_window_attention = attention_or_nothing
+
+        def step():   # noqa: F811
+            for t in layer.parameters():
+                t.grad = None
+            xin.grad = None
+            with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+                out = layer(xin)
+            out.backward(gout)
+            return out
+
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0").random_(0, 255)
         dst = torch.empty_like(src)
@@ -190,6 +218,21 @@ def main():
         "op_tflops": op_tflops, "op_frac_of_bf16_peak": op_tflops / PEAK_BF16_TFLOPS,
     }
 
+    if args.config == "layer":
+        res["metric"] = "LaCT layer tokens/sec fwd+bwd at 760M shape, 1 GPU (projections and window attention included)"
+        res["config"].pop("algorithmic_gflop_per_step")
+        res.pop("op_tflops"); res.pop("op_frac_of_bf16_peak")
+        no_attention[0] = True      # the same steps without the attention branch
+        for _ in range(2):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        res["ttt_branch_ms_per_step"] = (time.perf_counter() - t0) / args.steps * 1e3
+        no_attention[0] = False
+
     traffic, step_traffic = load_traffic(args.config)
     # ---- per-kernel durations: the same K steps again with HIP events around every launch, on the stream
     #      the kernels run on (a second pass, so that the events do not perturb `value`)
@@ -231,7 +274,7 @@ def main():
                            "source": f"profiles/{args.config}_fwd_bwd_hbm_traffic_pmc.txt (FETCH_SIZE + WRITE_SIZE of every kernel of a step)"}
 
     # ---- CPU baseline: the oracle (a restatement of the reference's non-fused PyTorch op) on the host cores
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and args.config != "layer":
         cb = b if args.config == "c1" else min(b, 4)   # bounded sample: the first `cb` heads, forward + backward
         cpu = {n: inp[n][:cb].clone().requires_grad_(True) for n in names}
         gc = go[:cb].cpu()
