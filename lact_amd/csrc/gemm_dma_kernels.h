@@ -11,6 +11,7 @@ using TS_ROW = TileShape<256, 128, 2, 2>;   // token-row GEMMs, one accumulator:
 using TS_SQ = TileShape<128, 128, 2, 2>;    // small square GEMMs (Newton-Schulz) and 2-3 accumulator kernels
 using TS_BWD = TileShape<128, 64, 2, 2>;    // six accumulators (update backward): 64x32 per wave
 using TS_NS = TileShape<192, 192, 2, 2>;    // 384-multiple square GEMMs (Newton-Schulz at d = dh = 384): 96x96 per wave
+using TS_N96 = TileShape<128, 96, 4, 1>;    // Newton-Schulz of few 384-multiple matrices: 12 instead of 9 blocks per 384 x 384 matrix
 
 template <class TS> constexpr int row_stages() { return TS::BM == 128 ? 4 : 3; }
 

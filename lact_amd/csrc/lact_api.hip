@@ -526,17 +526,23 @@ struct Runner {
   static bool tiles_fit(int r, int c, int bm, int bn) {
     return r % bm == 0 && r % bn == 0 && c % bn == 0 && (r / bm) * (c / bn) <= 32;
   }
-  // Tile of the fused kernel for a batch: 0 = 192 x 192, 1 = 128 x 128, 2 = 128 x 64, -1 = none fits.
+  // Tile of the fused kernel for a batch: 0 = 192 x 192, 1 = 128 x 128, 2 = 128 x 64, 3 = 128 x 96, -1 = none fits.
   // 192 x 192 when the matrices fill at least half the chip with it, else 128 x 128 (more, smaller blocks), and
-  // 128 x 64 when even those leave most of the chip idle -- as long as the groups dealt to one XCD (a matrix's
-  // blocks share an XCD) still find a compute unit each there.
+  // 128 x 64 or 128 x 96 when even those leave most of the chip idle -- as long as the groups dealt to one XCD (a
+  // matrix's blocks share an XCD) still find a compute unit each there.
   static int ns_fused_tile(const NsBatch& B) {
     const bool f192 = tiles_fit(B.r, B.c, 192, 192), f128 = tiles_fit(B.r, B.c, 128, 128), f64 = tiles_fit(B.r, B.c, 128, 64);
+    const bool f96 = tiles_fit(B.r, B.c, 128, 96);
     if (f192 && (!f128 || B.n * (B.r / 192) * (B.c / 192) >= 128)) return 0;
     const int per_xcd = (B.n + 7) / 8;
+    const bool sparse128 = !f128 || B.n * (B.r / 128) * (B.c / 128) < 128;
     if (f64) {
       const int nbm64 = (B.r / 128) * (B.c / 64);
-      if (per_xcd * nbm64 <= 32 && (!f128 || B.n * (B.r / 128) * (B.c / 128) < 128)) return 2;
+      if (per_xcd * nbm64 <= 32 && sparse128) return 2;
+    }
+    if (f96) {
+      const int nbm96 = (B.r / 128) * (B.c / 96);
+      if (per_xcd * nbm96 <= 32 && sparse128) return 3;
     }
     if (f128) return 1;
     return f192 ? 0 : -1;
@@ -546,6 +552,7 @@ struct Runner {
       case 0: return (B.r / 192) * (B.c / 192);
       case 1: return (B.r / 128) * (B.c / 128);
       case 2: return (B.r / 128) * (B.c / 64);
+      case 3: return (B.r / 128) * (B.c / 96);
       default: return 0;
     }
   }
@@ -604,6 +611,7 @@ struct Runner {
       case 0: launch_ns_fused_ts<TS_NS, BWD>(p, B); break;
       case 1: launch_ns_fused_ts<TS_SQ, BWD>(p, B); break;
       case 2: launch_ns_fused_ts<TS_BWD, BWD>(p, B); break;
+      case 3: launch_ns_fused_ts<TS_N96, BWD>(p, B); break;
       default: break;
     }
   }

@@ -1107,7 +1107,7 @@ def test_stream_overlap_is_bit_identical(prenorm):
     assert torch.equal(on[0][0], on[2][0]) and all(torch.equal(on[0][1][n], on[2][1][n]) for n in on[0][1])
 
 
-@pytest.mark.parametrize("b,d,dh", [(5, 384, 192), (2, 384, 384), (3, 256, 128),
+@pytest.mark.parametrize("b,d,dh", [(5, 384, 192), (2, 384, 384), (4, 384, 384), (3, 256, 128),
                                     (2, 768, 1536)])   # the video model's head: 32 blocks per matrix, a whole XCD per group
 def test_fused_newton_schulz_is_bit_identical(b, d, dh):
     """All Newton-Schulz iterations of an update as one kernel with per-matrix barriers (rows, columns multiples
@@ -1117,7 +1117,8 @@ def test_fused_newton_schulz_is_bit_identical(b, d, dh):
     say("fused Newton-Schulz on/off", b, d, dh)
     from lact_amd import _lib
     # (5, 384, 192): w1 is held transposed ([192, 384]), 15 matrices = a partial group of 8, 192-tiles;
-    # (2, 384, 384): few matrices -> 128-tiles, 9 blocks per matrix;  (3, 256, 128): only 128-tiles fit
+    # (2, 384, 384), (4, 384, 384): few matrices -> 128 x 96 tiles, 12 blocks per matrix, one or two groups per XCD;
+    # (3, 256, 128): only 128-tiles fit
     L, C = 3 * 256, 256
     inp = problem(b, L, d, dh, seed=91, act=torch.bfloat16)
     go = torch.randn(b, L, d, generator=torch.Generator().manual_seed(6)).bfloat16().to(DEV)
