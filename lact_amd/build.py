@@ -13,6 +13,15 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     # packed-fp32 VALU forms are kept out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # A multiply and an add fuse only where one source expression writes them together.  HIP's default ("fast") also
+    # fuses across statements and inlined calls, i.e. through __fmul_rn / __fadd_rn, which are plain operators in the
+    # HIP headers: whether a product that the reference rounds as a tensor of its own (a * X before + B @ X,
+    # ttt_operation.py:62; M * m before dw +, :174-176) got its own rounding then depended on how the surrounding
+    # kernel was inlined -- the fused and the unfused Newton-Schulz backward differed in exactly that.
+    "-ffp-contract=on",
+    # the copy engine sets m0 in its own asm statements and names it as clobbered; no compiler-generated code in these
+    # kernels uses m0 (no LDS-DMA builtins, no register-indexed moves, no messages)
+    "-Wno-inline-asm",
 ]
 
 

@@ -558,10 +558,27 @@ struct Runner {
   }
   // The fused kernel's groups must be resident as a whole, one block per compute unit, on a device that deals its
   // workgroups to 8 dies of 32 compute units: anything else (a partitioned or smaller device) takes the unfused launches.
-  bool ns_fused_ok(const NsBatch& B) const {
-    if (!g_fused_ns || !side || !kNsBf16 || P.S < 1 || P.S > NS_FUSED_MAX_STEPS) return false;
+  bool ns_fusable(const NsBatch& B) const {
+    if (!side || !kNsBf16 || P.S < 1 || P.S > NS_FUSED_MAX_STEPS) return false;
     if (side->cus < 256) return false;
     return ns_fused_tile(B) >= 0;
+  }
+  bool ns_fused_ok(const NsBatch& B) const { return g_fused_ns && ns_fusable(B); }
+  // The unfused launches of a batch the fused kernel could take sum the dot product of the normalisation's backward
+  // over the fused kernel's tiles, in its order: switching LACT_OPT_FUSED_NEWTON_SCHULZ then changes no bit.
+  bool ns_dot_by_tiles() const { return P.muon && P.nsb.size() == 1 && ns_fusable(P.nsb[0]); }
+  template <class TS>
+  void launch_ns_dot_tiles_ts(const NsTileDotParams& q, const NsBatch& B) {
+    LACT_LAUNCH("k_ns_bwd_dot_tiles", "k_ns_bwd_dot", 0.0, (k_ns_bwd_dot_tiles<TS>), dim3((B.r / TS::BM) * (B.c / TS::BN), B.n), dim3(DMA_THREADS), s, q);
+  }
+  void launch_ns_dot_tiles(const NsTileDotParams& q, const NsBatch& B) {
+    switch (ns_fused_tile(B)) {
+      case 0: launch_ns_dot_tiles_ts<TS_NS>(q, B); break;
+      case 1: launch_ns_dot_tiles_ts<TS_SQ>(q, B); break;
+      case 2: launch_ns_dot_tiles_ts<TS_BWD>(q, B); break;
+      case 3: launch_ns_dot_tiles_ts<TS_N96>(q, B); break;
+      default: break;
+    }
   }
   // every batch runs fused (and at least one iteration): the Frobenius normalisation is the fused kernel's first stage
   bool ns_all_fused() const {
@@ -1422,7 +1439,15 @@ struct Runner {
           }
         }
         cur = P.S & 1;
-        if (!dot_in_kernel) {
+        if (!dot_in_kernel && ns_dot_by_tiles()) {
+          if constexpr (kNsBf16) {
+            const NsBatch& B = P.nsb[0];
+            NsTileDotParams q;
+            q.gx = scr<float>(P.t_gxf[cur]) + B.xoff; q.g16 = reinterpret_cast<const uint16_t*>(g16(u)) + B.xoff;
+            q.dot_part = scr<float>(P.t_dot); q.r = B.r; q.c = B.c;
+            launch_ns_dot_tiles(q, B);
+          }
+        } else if (!dot_in_kernel) {
           NsDotParams dp;
           dp.g = P.g; dp.gx0 = scr<float>(P.t_gxf[cur]); dp.g16 = g16(u); dp.dot_part = scr<float>(P.t_dot);
           LACT_LAUNCH("k_ns_bwd_dot", "k_ns_bwd_dot", 0.0, (k_ns_bwd_dot<TN>), dim3(P.nblk, P.g.ns_count()), dim3(256), s, dp);
@@ -1434,7 +1459,7 @@ struct Runner {
         memset(&p, 0, sizeof(p));
         p.g = P.g; p.muon = P.muon;
         p.gx0 = scr<float>(P.t_gxf[cur]); p.g16 = P.muon ? (const void*)g16(u) : nullptr; p.norms = norms(u);
-        p.dot_part = scr<float>(P.t_dot); p.nparts = (P.muon && dot_in_kernel) ? ns_fused_nbm(P.nsb[0]) : P.nblk;
+        p.dot_part = scr<float>(P.t_dot); p.nparts = (P.muon && (dot_in_kernel || ns_dot_by_tiles())) ? ns_fused_nbm(P.nsb[0]) : P.nblk;
         p.gw_hat = gwhat; p.cr = (P.muon && d.muon_replaces_weight) ? 1.f : 0.f;
         p.gm_carry = (P.momentum && (u > 0 || gm_valid)) ? gmcarry : nullptr; p.carry_valid = gm_valid;
         p.carry_write = u > 0;

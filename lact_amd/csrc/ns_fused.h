@@ -125,6 +125,54 @@ __device__ __forceinline__ void ns_term(RowGemmTerm& t, const void* A, int lda, 
   t.A = A; t.lda = lda; t.bsA = bsA; t.B = B; t.ldb = ldb; t.bsB = bsB; t.K = K;
 }
 
+// <gx, g16> over one TS::BM x TS::BN tile whose first element is at offset zo of both arrays (row stride c): every thread
+// takes the granules of 8 elements threadIdx.x, threadIdx.x + DMA_THREADS, ... and keeps what it read (ga, gb: the fp32
+// values, gi: the bf16 ones).  Returns this thread's partial sum.  The fused kernel and k_ns_bwd_dot_tiles both sum a
+// tile through this one function and block_sum, so the two paths produce the same bits.
+template <class TS, int NG>
+__device__ __forceinline__ float ns_tile_dot(const float* gx, const uint16_t* g16, size_t zo, int c, float4 (&ga)[NG], float4 (&gb)[NG], uint4 (&gi)[NG]) {
+  constexpr int GR = TS::BN / 8;
+  static_assert(NG == (TS::BM * GR + DMA_THREADS - 1) / DMA_THREADS, "granules per thread");
+  float dot = 0.f;
+#pragma unroll
+  for (int t = 0; t < NG; ++t) {
+    const int id = threadIdx.x + t * DMA_THREADS;
+    if (id < TS::BM * GR) {
+      const size_t o = zo + (size_t)(id / GR) * c + (id % GR) * 8;
+      ga[t] = *reinterpret_cast<const float4*>(gx + o);
+      gb[t] = *reinterpret_cast<const float4*>(gx + o + 4);
+      gi[t] = *reinterpret_cast<const uint4*>(g16 + o);
+      const uint32_t w[4] = {gi[t].x, gi[t].y, gi[t].z, gi[t].w};
+      dot += ga[t].x * __uint_as_float(w[0] << 16) + ga[t].y * __uint_as_float(w[0] & 0xffff0000u) +
+             ga[t].z * __uint_as_float(w[1] << 16) + ga[t].w * __uint_as_float(w[1] & 0xffff0000u) +
+             gb[t].x * __uint_as_float(w[2] << 16) + gb[t].y * __uint_as_float(w[2] & 0xffff0000u) +
+             gb[t].z * __uint_as_float(w[3] << 16) + gb[t].w * __uint_as_float(w[3] & 0xffff0000u);
+    }
+  }
+  return dot;
+}
+
+// The partial dots of the Frobenius normalisation's backward as the fused backward kernel forms them (one per tile of
+// the fused kernel's tiling, summed in its order), for the unfused launches: the two paths then hand the same bits
+// to everything downstream.  Grid (tiles per matrix, matrices); matrices are [r, c] one after the other.
+struct NsTileDotParams {
+  const float* gx; const uint16_t* g16; float* dot_part;
+  int r, c;
+};
+template <class TS>
+__global__ __launch_bounds__(DMA_THREADS) void k_ns_bwd_dot_tiles(const NsTileDotParams p) {
+  __shared__ float red[16];
+  constexpr int GR = TS::BN / 8, NG = (TS::BM * GR + DMA_THREADS - 1) / DMA_THREADS;
+  const int tc = p.c / TS::BN, member = blockIdx.x, z = blockIdx.y;
+  const int rx = member / tc, ry = member % tc;
+  const size_t zo = (size_t)z * p.r * p.c + (size_t)rx * TS::BM * p.c + ry * TS::BN;
+  float4 ga[NG], gb[NG];
+  uint4 gi[NG];
+  float dot = ns_tile_dot<TS>(p.gx, p.g16, zo, p.c, ga, gb, gi);
+  dot = block_sum(dot, red);
+  if (threadIdx.x == 0) p.dot_part[(size_t)z * gridDim.x + member] = dot;
+}
+
 // BWD = false: S iterations  A = X X^T;  B = b A + c A A;  X' = a X + B X
 // BWD = true:  the same iterations backwards:  Sg = G X^T + X G^T;  H = b Sg + c (Sg A + A Sg);  G' = a G + B G + H X
 // TS: 192 x 192 tiles, or 128 x 128 / 128 x 64 when there are too few matrices to fill the chip with the large tile.
@@ -274,25 +322,10 @@ __global__ __launch_bounds__(DMA_THREADS) void k_ns_fused(const NsFusedParams p)
     const size_t zo = (size_t)z * p.r * p.c + (size_t)rx * TS::BM * p.c + ry * TS::BN;
     float4 ga[NG], gb[NG];
     uint4 gi[NG];
-    float dot = 0.f;
     // No fence: this tile of gx was written by this very block in the last stage (and in every second stage before),
     // and the waves of a compute unit share its vector L1, which their own stores keep current.  The same holds for
     // every auxiliary tile the blending epilogues read (always the block's own tile of a buffer it wrote itself).
-#pragma unroll
-    for (int t = 0; t < NG; ++t) {
-      const int id = threadIdx.x + t * DMA_THREADS;
-      if (id < TS::BM * GR) {
-        const size_t o = zo + (size_t)(id / GR) * p.c + (id % GR) * 8;
-        ga[t] = *reinterpret_cast<const float4*>(gx + o);
-        gb[t] = *reinterpret_cast<const float4*>(gx + o + 4);
-        gi[t] = *reinterpret_cast<const uint4*>(p.g16 + o);
-        const uint32_t w[4] = {gi[t].x, gi[t].y, gi[t].z, gi[t].w};
-        dot += ga[t].x * __uint_as_float(w[0] << 16) + ga[t].y * __uint_as_float(w[0] & 0xffff0000u) +
-               ga[t].z * __uint_as_float(w[1] << 16) + ga[t].w * __uint_as_float(w[1] & 0xffff0000u) +
-               gb[t].x * __uint_as_float(w[2] << 16) + gb[t].y * __uint_as_float(w[2] & 0xffff0000u) +
-               gb[t].z * __uint_as_float(w[3] << 16) + gb[t].w * __uint_as_float(w[3] & 0xffff0000u);
-      }
-    }
+    float dot = ns_tile_dot<TS>(gx, p.g16, zo, p.c, ga, gb, gi);
     dot = block_sum(dot, reinterpret_cast<float*>(smem));
     if (threadIdx.x == 0) p.dot_part[(size_t)z * nbm + member] = dot;
     if (p.gc) {
