@@ -1,9 +1,11 @@
 """Benchmark of the TTT operation on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1|c2|c3|c4|layer] [--no-cpu-baseline]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--repeats R] [--config c1|c2|c3|c4|layer] [--no-cpu-baseline]
 
 One step = forward + backward of block_causal_lact_swiglu over one batch of seeded synthetic input
-that is resident in HBM before the timed region.  Prints one JSON line (metric: tokens/s, tokens = B*L).
+that is resident in HBM before the timed region.  After W warm-up steps, R regions of exactly K steps are timed
+(each between two device synchronisations); `value` comes from the median region.  Prints one JSON line
+(metric: tokens/s, tokens = B*L); for config c1 the line also carries short runs of c2, c3 and c4 (`other_configs`).
 """
 import argparse
 import ctypes
@@ -102,6 +104,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", default="c1", choices=sorted(CONFIGS))
+    ap.add_argument("--repeats", type=int, default=5, help="timed regions of --steps steps each; the median region is reported")
+    ap.add_argument("--no-other-configs", action="store_true", help="config c1 only: skip the short runs of c2, c3 and c4")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-profile", action="store_true")
     ap.add_argument("--no-overlap", action="store_true",
@@ -124,56 +128,100 @@ def main():
     from lact_amd import _lib
     from oracle import lact_oracle as O
 
-    B, H, L, d, dh, C, seed, text = CONFIGS[args.config]
-    b = B * H
-    inp = O.make_inputs(b, L, d, dh, seed=seed, act_dtype=torch.bfloat16, distinct_heads=H, momentum_value=0.9)
     order = ("w0", "w1", "w2", "q", "k", "v", "lr0", "lr1", "lr2")
     names = list(order) + ["momentum"]
-    dev = {n: inp[n].to("cuda:0").requires_grad_(True) for n in names}
-    go = torch.randn(b, L, d, generator=torch.Generator().manual_seed(seed + 1)).bfloat16().to("cuda:0")
 
-    def step():
-        for t in dev.values():
-            t.grad = None
-        out = lact_amd.block_causal_lact_swiglu(*[dev[n] for n in order], C, True, dev["momentum"])
-        out.backward(go)
-        return out
+    def build_workload(cfg):
+        """The step function of a configuration (inputs resident in HBM) and what describes it."""
+        B, H, L, d, dh, C, seed, text = CONFIGS[cfg]
+        b = B * H
+        w = {"B": B, "H": H, "L": L, "d": d, "dh": dh, "C": C, "b": b, "seed": seed, "text": text}
+        if cfg == "c3":
+            import math as _m
+            from lact_amd import nvs
+            inp3 = O.make_inputs(b, L, d, dh, seed=seed, act_dtype=torch.bfloat16, momentum_value=None)
+            for n in ("w0", "w1", "w2"):      # transposed layout and sqrt(2) gain of lact_nvs/lact_ttt.py:184-193
+                inp3[n] = (inp3[n] * _m.sqrt(2.0)).transpose(1, 2).contiguous()
+            dev3 = [inp3[n].to("cuda:0") for n in order]
+            program = [nvs.TTTOperator(0, C, True, False), nvs.TTTOperator(C, L, False, True)]
 
-    if args.config == "c3":
-        import math as _m
-        from lact_amd import nvs
-        inp3 = O.make_inputs(b, L, d, dh, seed=seed, act_dtype=torch.bfloat16, momentum_value=None)
-        for n in ("w0", "w1", "w2"):      # transposed layout and sqrt(2) gain of lact_nvs/lact_ttt.py:184-193
-            inp3[n] = (inp3[n] * _m.sqrt(2.0)).transpose(1, 2).contiguous()
-        dev3 = [inp3[n].to("cuda:0") for n in order]
-        program = [nvs.TTTOperator(0, C, True, False), nvs.TTTOperator(C, L, False, True)]
+            def step():
+                with torch.no_grad():
+                    return nvs.fast_weight_swish_glu_weight_norm_mini_batch_apply(*dev3, program, 5)[0]
+            r_, c_ = min(d, dh), max(d, dh)   # forward only; apply on L - C tokens, one update on C tokens
+            w["flops"] = b * (6.0 * d * dh * (L - C) + 12.0 * d * dh * C + 3.0 * 5 * (4.0 * r_ * r_ * c_ + 2.0 * r_ ** 3))
+            w.update(step=step, inp3=inp3, program=program)
+            return w
+        if cfg == "layer":
+            from lact_amd import layers
+            torch.manual_seed(seed)
+            layer = layers.CausalLaCTSwiGLUWithSlidingWindowAttn(dim=H * d, head_dim=d, attn_head_dim=128, lact_chunk_size=C,
+                                                                 window_size=2048).to("cuda:0")
+            xin = torch.randn(B, L, H * d, generator=torch.Generator().manual_seed(seed)).to("cuda:0").requires_grad_(True)
+            gout = torch.randn(B, L, H * d, generator=torch.Generator().manual_seed(seed + 1)).bfloat16().to("cuda:0")
+            no_attention = [False]
+            real_attention = layers.sliding_window_attention
 
-        def step():   # noqa: F811
-            with torch.no_grad():
-                return nvs.fast_weight_swish_glu_weight_norm_mini_batch_apply(*dev3, program, 5)[0]
+            def attention_or_nothing(q_, k_, v_, window):   # the TTT branch alone: attention replaced by its value input
+                return v_ if no_attention[0] else real_attention(q_, k_, v_, window)
+            layers.sliding_window_attention = attention_or_nothing
 
-    if args.config == "layer":
-        from lact_amd import layers
-        torch.manual_seed(seed)
-        layer = layers.CausalLaCTSwiGLUWithSlidingWindowAttn(dim=H * d, head_dim=d, attn_head_dim=128, lact_chunk_size=C,
-                                                             window_size=2048).to("cuda:0")
-        xin = torch.randn(B, L, H * d, generator=torch.Generator().manual_seed(seed)).to("cuda:0").requires_grad_(True)
-        gout = torch.randn(B, L, H * d, generator=torch.Generator().manual_seed(seed + 1)).bfloat16().to("cuda:0")
-        no_attention = [False]
-        real_attention = layers.sliding_window_attention
+            def step():
+                for t in layer.parameters():
+                    t.grad = None
+                xin.grad = None
+                with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+                    out = layer(xin)
+                out.backward(gout)
+                return out
+            w.update(step=step, no_attention=no_attention, flops=None)
+            return w
+        inp = O.make_inputs(b, L, d, dh, seed=seed, act_dtype=torch.bfloat16, distinct_heads=H, momentum_value=0.9)
+        dev = {n: inp[n].to("cuda:0").requires_grad_(True) for n in names}
+        go = torch.randn(b, L, d, generator=torch.Generator().manual_seed(seed + 1)).bfloat16().to("cuda:0")
 
-        def attention_or_nothing(q_, k_, v_, window):   # the TTT branch alone: attention replaced by its value input
-            return v_ if no_attention[0] else real_attention(q_, k_, v_, window)
-        layers.sliding_window_attention = attention_or_nothing
-
-        def step():   # noqa: F811
-            for t in layer.parameters():
+        def step():
+            for t in dev.values():
                 t.grad = None
-            xin.grad = None
-            with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
-                out = layer(xin)
-            out.backward(gout)
+            out = lact_amd.block_causal_lact_swiglu(*[dev[n] for n in order], C, True, dev["momentum"])
+            out.backward(go)
             return out
+        w.update(step=step, inp=inp, go=go, flops=algorithmic_flops(b, L, d, dh, C))
+        return w
+
+    def time_steps(step, k):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(k):
+            step()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / k * 1e3
+
+    def kernel_profile(step, k):
+        """Per-launch durations of k more steps (HIP events on the launch stream, kernels one at a time)."""
+        Lb = _lib.lib()
+        Lb.lact_set_option(_lib.OPT_STREAM_OVERLAP, 0)
+        Lb.lact_profile_enable(1)
+        for _ in range(k):
+            step()
+        buf = ctypes.create_string_buffer(1 << 20)
+        _lib.check(Lb.lact_profile_report(buf, len(buf)))
+        Lb.lact_profile_enable(0)
+        Lb.lact_set_option(_lib.OPT_STREAM_OVERLAP, 0 if args.no_overlap else 1)
+        rows = json.loads(buf.value.decode())
+        by_kernel = {}
+        for r in rows:
+            kk = by_kernel.setdefault(r["kernel"], {"launches": 0, "ms": 0.0, "flops": 0.0})
+            kk["launches"] += r["launches"]; kk["ms"] += r["ms"]; kk["flops"] += r["flops"]
+        total_ms = sum(kk["ms"] for kk in by_kernel.values())
+        dom_name, dom = max(((n, kk) for n, kk in by_kernel.items() if kk["flops"] > 0), key=lambda x: x[1]["ms"])
+        avg_ms = dom["ms"] / dom["launches"]
+        achieved = dom["flops"] / dom["launches"] / (avg_ms * 1e-3) / 1e12
+        return rows, total_ms, dom_name, dom, avg_ms, achieved
+
+    W = build_workload(args.config)
+    B, H, L, d, dh, C, b, seed, text = (W[n] for n in ("B", "H", "L", "d", "dh", "C", "b", "seed", "text"))
+    step = W["step"]
 
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0").random_(0, 255)
@@ -195,66 +243,41 @@ def main():
         _lib.lib().lact_set_option(_lib.OPT_STREAM_OVERLAP, 0)
     for _ in range(args.warmup):
         step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    ms_per_step = dt / args.steps * 1e3
-    tokens_per_s = B * L * args.steps / dt
-    flops = algorithmic_flops(b, L, d, dh, C)
-    if args.config == "c3":   # forward only; apply on L - C tokens, one update on C tokens
-        r_, c_ = min(d, dh), max(d, dh)
-        flops = b * (6.0 * d * dh * (L - C) + 12.0 * d * dh * C + 3.0 * 5 * (4.0 * r_ * r_ * c_ + 2.0 * r_ ** 3))
-    op_tflops = flops / (ms_per_step * 1e-3) / 1e12
+    # `repeats` timed regions of exactly `steps` steps each, every one bracketed by a device synchronisation; the
+    # reported step time is the median region's (a region is a few tens of milliseconds: one scheduler hiccup on the
+    # host would otherwise move the figure by percent).  All regions are listed in `ms_per_step_repeats`.
+    reps_ms = [time_steps(step, args.steps) for _ in range(max(1, args.repeats))]
+    ms_per_step = sorted(reps_ms)[len(reps_ms) // 2]
+    tokens_per_s = B * L / (ms_per_step * 1e-3)
+    flops = W["flops"]
 
     res = {
         "metric": "TTT-layer tokens/sec fwd+bwd at 760M shape, 1 GPU; MFMA util % of bf16 peak",
         "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic (seeded N(0,1) q,k,v; L2-normalised q,k; random-init fast weights)",
-        "config": {"workload": text, "tokens_per_step": B * L, "algorithmic_gflop_per_step": flops / 1e9},
-        "op_tflops": op_tflops, "op_frac_of_bf16_peak": op_tflops / PEAK_BF16_TFLOPS,
+        "config": {"workload": text, "tokens_per_step": B * L},
+        "ms_per_step_repeats": reps_ms,
     }
+    if flops is not None:
+        op_tflops = flops / (ms_per_step * 1e-3) / 1e12
+        res["config"]["algorithmic_gflop_per_step"] = flops / 1e9
+        res["op_tflops"] = op_tflops
+        res["op_frac_of_bf16_peak"] = op_tflops / PEAK_BF16_TFLOPS
 
     if args.config == "layer":
         res["metric"] = "LaCT layer tokens/sec fwd+bwd at 760M shape, 1 GPU (projections and window attention included)"
-        res["config"].pop("algorithmic_gflop_per_step")
-        res.pop("op_tflops"); res.pop("op_frac_of_bf16_peak")
-        no_attention[0] = True      # the same steps without the attention branch
+        W["no_attention"][0] = True      # the same steps without the attention branch
         for _ in range(2):
             step()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            step()
-        torch.cuda.synchronize()
-        res["ttt_branch_ms_per_step"] = (time.perf_counter() - t0) / args.steps * 1e3
-        no_attention[0] = False
+        res["ttt_branch_ms_per_step"] = time_steps(step, args.steps)
+        W["no_attention"][0] = False
 
     traffic, step_traffic = load_traffic(args.config)
     # ---- per-kernel durations: the same K steps again with HIP events around every launch, on the stream
     #      the kernels run on (a second pass, so that the events do not perturb `value`)
     if not args.no_kernel_profile:
-        Lb = _lib.lib()
-        Lb.lact_set_option(_lib.OPT_STREAM_OVERLAP, 0)      # one kernel at a time: the duration of a launch is that kernel's own
-        Lb.lact_profile_enable(1)
-        for _ in range(args.steps):
-            step()
-        buf = ctypes.create_string_buffer(1 << 20)
-        _lib.check(Lb.lact_profile_report(buf, len(buf)))
-        Lb.lact_profile_enable(0)
-        Lb.lact_set_option(_lib.OPT_STREAM_OVERLAP, 0 if args.no_overlap else 1)
-        rows = json.loads(buf.value.decode())
-        by_kernel = {}
-        for r in rows:
-            k = by_kernel.setdefault(r["kernel"], {"launches": 0, "ms": 0.0, "flops": 0.0})
-            k["launches"] += r["launches"]; k["ms"] += r["ms"]; k["flops"] += r["flops"]
-        total_ms = sum(k["ms"] for k in by_kernel.values())
-        dom_name, dom = max(((n, k) for n, k in by_kernel.items() if k["flops"] > 0), key=lambda x: x[1]["ms"])
-        avg_ms = dom["ms"] / dom["launches"]
-        achieved = dom["flops"] / dom["launches"] / (avg_ms * 1e-3) / 1e12
+        rows, total_ms, dom_name, dom, avg_ms, achieved = kernel_profile(step, args.steps)
         res["roofline"] = {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                            "frac": achieved / PEAK_BF16_TFLOPS,
                            "traffic": traffic.get(dom_name),
@@ -276,14 +299,15 @@ def main():
     # ---- CPU baseline: the oracle (a restatement of the reference's non-fused PyTorch op) on the host cores
     if not args.no_cpu_baseline and args.config != "layer":
         cb = b if args.config == "c1" else min(b, 4)   # bounded sample: the first `cb` heads, forward + backward
-        cpu = {n: inp[n][:cb].clone().requires_grad_(True) for n in names}
-        gc = go[:cb].cpu()
+        if args.config != "c3":
+            cpu = {n: W["inp"][n][:cb].clone().requires_grad_(True) for n in names}
+            gc = W["go"][:cb].cpu()
         t0 = time.perf_counter()
         reps = 0
         while reps < 1 or (time.perf_counter() - t0 < 12.0 and reps < 40):
             if args.config == "c3":   # forward only, as the GPU leg
                 with torch.no_grad():
-                    O.fast_weight_swish_glu_weight_norm_mini_batch_apply(*[inp3[n][:cb] for n in order], program, 5,
+                    O.fast_weight_swish_glu_weight_norm_mini_batch_apply(*[W["inp3"][n][:cb] for n in order], W["program"], 5,
                                                                          num=O.Numerics(autocast=True))
             else:
                 for t in cpu.values():
@@ -296,6 +320,30 @@ def main():
                                "kind": "port",
                                "sample": f"first {cb} of {b} heads of the same workload, {'fwd' if args.config == 'c3' else 'fwd+bwd'}, {reps} run(s), "
                                          f"{ct:.2f} s each; tokens scaled by {cb}/{b}; host has {os.cpu_count()} logical CPUs"}
+    # ---- the other BASELINE configurations, timed the same way (median of three regions), each with its dominant kernel
+    if args.config == "c1" and not args.no_other_configs:
+        del W, step
+        torch.cuda.empty_cache()
+        res["other_configs"] = {}
+        for cfg in ("c2", "c3", "c4"):
+            Wc = build_workload(cfg)
+            for _ in range(3):
+                Wc["step"]()
+            k = max(5, args.steps // 2)
+            r3 = [time_steps(Wc["step"], k) for _ in range(3)]
+            ms = sorted(r3)[1]
+            tf = Wc["flops"] / (ms * 1e-3) / 1e12
+            entry = {"workload": Wc["text"], "ms_per_step": ms, "tokens_per_s": Wc["B"] * Wc["L"] / (ms * 1e-3), "steps": k,
+                     "ms_per_step_repeats": r3, "algorithmic_gflop_per_step": Wc["flops"] / 1e9, "op_tflops": tf,
+                     "op_frac_of_bf16_peak": tf / PEAK_BF16_TFLOPS}
+            if not args.no_kernel_profile:
+                _, total_ms_c, dom_name_c, dom_c, avg_ms_c, achieved_c = kernel_profile(Wc["step"], k)
+                entry["dominant_kernel"] = {"kernel": dom_name_c, "avg_launch_ms": avg_ms_c, "launches_per_step": dom_c["launches"] / k,
+                                            "achieved_tflops": achieved_c, "frac": achieved_c / PEAK_BF16_TFLOPS,
+                                            "share_of_kernel_time": dom_c["ms"] / total_ms_c}
+            res["other_configs"][cfg] = entry
+            del Wc
+            torch.cuda.empty_cache()
     print(json.dumps(res))
 
 

@@ -32,6 +32,14 @@ def _ar_steps(seq_len, q_len, mini_batch_size, update_length, update_every, num_
     return tuple(steps)
 
 
+def _scaled(lr, w_scale: float):
+    """The reference forms (k * lr) * w_scale, left to right (ar_lact_swa_repeat.py:134-138); the kernels take one
+    per-token factor, so lr * w_scale is folded first.  The two agree bit for bit when w_scale is a power of two --
+    the layer's only value is 1.0 (ar_lact_swa_repeat.py:629) -- and otherwise differ by one fp32 rounding in front of
+    the bf16 cast of the GEMM operand."""
+    return lr if w_scale == 1.0 else lr * w_scale
+
+
 def ar_fast_weight_swish_glu_weight_norm_mini_batch_with_momentum(
         w0, w1, w2, q, k, v, lr0, lr1, lr2, w_scale: float, num_repeat: int = 1, mini_batch_size: int = -1,
         update_length: int = -1, update_every: int = -1, use_moun: bool = False, num_moun_iters: int = 3,
@@ -40,7 +48,7 @@ def ar_fast_weight_swish_glu_weight_norm_mini_batch_with_momentum(
     prog = Program(steps=_ar_steps(k.shape[1], q.shape[1], mini_batch_size, update_length, update_every, num_repeat),
                    out_len=q.shape[1], ns_coeffs=(NS_CLASSIC,) * num_moun_iters if use_moun else None,
                    weight_norm=weight_norm, ns_mode=ops._ns_mode(q))
-    out, ws, _ = run_program(prog, w0, w1, w2, q, k, v, lr0 * w_scale, lr1 * w_scale, lr2 * w_scale,
+    out, ws, _ = run_program(prog, w0, w1, w2, q, k, v, _scaled(lr0, w_scale), _scaled(lr1, w_scale), _scaled(lr2, w_scale),
                              fw_momentum if use_momentum else None)
     return (out,) + tuple(ws)
 
@@ -64,7 +72,7 @@ def ar_fast_weight_swish_glu_weight_norm_mini_batch_inference(
     prog = Program(steps=tuple(steps), out_len=q.shape[1],
                    ns_coeffs=(NS_CLASSIC,) * num_moun_iters if use_moun else None,
                    weight_norm=weight_norm, ns_mode=ops._ns_mode(q))
-    out, ws, _ = run_program(prog, w0, w1, w2, q, k, v, lr0 * w_scale, lr1 * w_scale, lr2 * w_scale, None)
+    out, ws, _ = run_program(prog, w0, w1, w2, q, k, v, _scaled(lr0, w_scale), _scaled(lr1, w_scale), _scaled(lr2, w_scale), None)
     return (out,) + tuple(ws)
 
 
@@ -83,7 +91,7 @@ def ar_fast_weight_swish_glu_weight_norm_mini_batch_inference_with_momentum(
                    ns_coeffs=(NS_CLASSIC,) * num_moun_iters if use_moun else None,
                    weight_norm=weight_norm, ns_mode=ops._ns_mode(q))
     state = (dw0_momentum, dw1_momentum, dw2_momentum) if (use_momentum and dw0_momentum is not None) else None
-    out, ws, ms = run_program(prog, w0, w1, w2, q, k, v, lr0 * w_scale, lr1 * w_scale, lr2 * w_scale,
+    out, ws, ms = run_program(prog, w0, w1, w2, q, k, v, _scaled(lr0, w_scale), _scaled(lr1, w_scale), _scaled(lr2, w_scale),
                               fw_momentum if use_momentum else None, momentum_state=state if updates else None)
     if not use_momentum:
         ms = (dw0_momentum, dw1_momentum, dw2_momentum)           # handed through untouched (:339)

@@ -362,6 +362,7 @@ __global__ __launch_bounds__(DMA_THREADS) void k_update_hidden_dma(const HiddenD
   f32x16 a02[2][TS::TM][TS::TN], a1[1][TS::TM][TS::TN];
   three_acc_mainloop<TS>(pp, smem, m0, n0, z, a02, a1);
   using SB = StageTile<TS, 2>;
+  static_assert(4 * SB::BYTES <= 160 * 1024, "four staged tiles must fit the LDS (the launch asks for at least that much)");
   char* s0 = smem + SB::lane_base(); char* s1 = s0 + SB::BYTES; char* s2 = s0 + 2 * SB::BYTES; char* s3 = s0 + 3 * SB::BYTES;
   const int ntm = threadIdx.x < TS::THREADS ? TS::TM : 0;   // the loader waves own no fragments
   const bool keep = p.O3 != nullptr;

@@ -238,9 +238,10 @@ struct Plan {
   size_t mat3 = 0;  // 3*b*elems
   // saved
   size_t s_n0, s_wf, s_wc, s_main, s_d, s_min, s_mbar, s_u, s_g16, s_norms, s_xb, s_ab, s_bb, saved_bytes;
-  // Kept for the backward on the asynchronous-copy path: per update, eight token-major arrays [b][T][dh] -- the three
-  // lr-scaled hidden-side operands the backward's GEMMs read, the three rounded pre-activations they came from, and
-  // the two unscaled operands of the forward's dw0 / dw2 reductions (which scale k instead).
+  // Kept for the backward on the asynchronous-copy path: per update, six token-major arrays [b][T][dh] -- the three
+  // lr-scaled hidden-side operands the backward's GEMMs read and the three rounded pre-activations they came from.
+  // (The two unscaled operands of the forward's dw0 / dw2 reductions, which scale k instead, are read by the forward's
+  // own token reduction only: they live in the call's scratch.)
   // 288 GB of HBM make keeping them cheaper than the three GEMMs that would recompute them.
   bool keep_pre = false;
   std::vector<size_t> s_pre;   // by update index
@@ -367,7 +368,7 @@ struct Plan {
       for (const auto& st : steps)
         if (st.kind == LACT_UPDATE) {
           pre_T.push_back(st.end - st.start);
-          s_pre.push_back(sv.take((size_t)8 * d.b * (st.end - st.start) * d.dh * esz));
+          s_pre.push_back(sv.take((size_t)6 * d.b * (st.end - st.start) * d.dh * esz));
         }
     saved_bytes = sv.off + 256;
 
@@ -665,7 +666,7 @@ struct Runner {
   TN* ab(int u, int it) const { return reinterpret_cast<TN*>(sv + P.s_ab) + ((size_t)u * std::max(1, P.S) + it) * sq3(); }
   TN* bb(int u, int it) const { return reinterpret_cast<TN*>(sv + P.s_bb) + ((size_t)u * std::max(1, P.S) + it) * sq3(); }
   T* h(int i) const { return reinterpret_cast<T*>(sc + hsel[i]); }
-  // kept array i (0..2: lr-scaled operands, 3..5: pre-activations, 6..7: unscaled operands 0 and 2) of update u; batch stride pre_bs(u)
+  // kept array i (0..2: lr-scaled operands, 3..5: pre-activations) of update u; batch stride pre_bs(u)
   T* pre(int u, int i) const { return reinterpret_cast<T*>(sv + P.s_pre[u]) + (size_t)i * d.b * P.pre_T[u] * d.dh; }
   long long pre_bs(int u) const { return (long long)P.pre_T[u] * d.dh; }
   static constexpr bool kBf16 = std::is_same<T, uint16_t>::value;
@@ -686,7 +687,7 @@ struct Runner {
       HiddenDmaParams q;
       q.h = hp;
       (void)ver;
-      constexpr int SM3 = cmax(DmaSmem<TS_SQ, 2, 3>::BYTES, 3 * StageTile<TS_SQ, 2>::BYTES);
+      constexpr int SM3 = cmax(DmaSmem<TS_SQ, 2, 3>::BYTES, 4 * StageTile<TS_SQ, 2>::BYTES);   // k_update_hidden_dma stages four tiles at a time
       constexpr int SM6 = cmax(DmaSmem<TS_BWD, 2, 3>::BYTES, 6 * StageTile<TS_BWD, 2>::BYTES);
       const TileMap m3 = make_tile_map(ceil_div(T_, TS_SQ::BM), ceil_div(d.dh, TS_SQ::BN), d.b);
       const TileMap m6 = make_tile_map(ceil_div(T_, TS_BWD::BM), ceil_div(d.dh, TS_BWD::BN), d.b);
@@ -965,7 +966,8 @@ struct Runner {
         T* z0 = h(0); T* z1 = h(1); T* z2 = h(2);
         long long zbs = hbs();
         if (P.keep_pre) {
-          z0 = pre(u, 6); z1 = pre(u, 1); z2 = pre(u, 7); zbs = pre_bs(u);
+          // the unscaled operands stay in scratch (each region holds b * Tcap * dh elements: room for this stride)
+          z0 = h(0); z1 = pre(u, 1); z2 = h(2); zbs = pre_bs(u);
           hp.O3 = pre(u, 3); hp.O4 = pre(u, 4); hp.O5 = pre(u, 5);
           hp.O6 = pre(u, 0); hp.O7 = pre(u, 2);
           hp.bso = zbs;

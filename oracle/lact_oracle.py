@@ -200,10 +200,11 @@ def swiglu_apply(w0, w1, w2, q, num: Numerics = Numerics()) -> torch.Tensor:
 
 
 def fast_weight_grads(w0, w1, w2, k, v, lr0, lr1, lr2, num: Numerics = Numerics(),
-                      cast_lr_operand: bool = True):
+                      cast_lr_operand: bool = True, w_scale: Optional[float] = None):
     """ttt_operation.py:147-168.  Returns (dw0, dw1, dw2), the lr-weighted descent direction of
     L = -sum_t <f_w(k_t), v_t>.  `cast_lr_operand=False` is the AR-video spelling
-    (ar_lact_swa_repeat.py:134-138), which leaves the lr-scaled operand in fp32 until the matmul."""
+    (ar_lact_swa_repeat.py:134-138), which leaves the lr-scaled operand in fp32 until the matmul and
+    multiplies by `w_scale` AFTER the learning rate: (k * lr) * w_scale."""
     kt = k.transpose(1, 2)          # [b, dk, l]
     vt = v.transpose(1, 2)          # [b, dv, l]
     g = num.mm(w0, kt)              # gate_before_act   [b, dh, l]
@@ -216,6 +217,8 @@ def fast_weight_grads(w0, w1, w2, k, v, lr0, lr1, lr2, num: Numerics = Numerics(
     r1 = hidden.transpose(1, 2) * lr1
     r0 = k * lr0
     r2 = k * lr2
+    if w_scale is not None:         # ar_lact_swa_repeat.py:134-138: left to right, the scale last
+        r1, r0, r2 = r1 * w_scale, r0 * w_scale, r2 * w_scale
     if cast_lr_operand:
         r1, r0, r2 = r1.type_as(vt), r0.type_as(dg), r2.type_as(dh2)
     dw1 = num.mm(vt, r1)
@@ -249,6 +252,7 @@ def run_program(w0, w1, w2, q, k, v, lr0, lr1, lr2, steps: Sequence[Step], *,
                 cast_lr_operand: bool = True,
                 out_rows: Optional[int] = None,
                 scatter_output: bool = True,
+                w_scale: Optional[float] = None,
                 stack_muon: bool = False,
                 eps_in_sqrt: bool = False,
                 momentum_state: Optional[Sequence[torch.Tensor]] = None):
@@ -280,7 +284,7 @@ def run_program(w0, w1, w2, q, k, v, lr0, lr1, lr2, steps: Sequence[Step], *,
             continue
         dw0, dw1, dw2 = fast_weight_grads(w0, w1, w2, k[:, s:e], v[:, s:e],
                                           lr0[:, s:e], lr1[:, s:e], lr2[:, s:e], num,
-                                          cast_lr_operand)
+                                          cast_lr_operand, w_scale)
         if mom is not None:                         # ttt_operation.py:170-179
             m = momentum[:, s:e].mean(dim=1, keepdim=True)
             dw0 = dw0 + mom[0] * m
@@ -458,7 +462,7 @@ def ar_fast_weight_swish_glu_weight_norm_mini_batch(w0, w1, w2, q, k, v, lr0, lr
     """ar_lact_swa_repeat.py:23-168 and, with momentum, ar_lact_swa_repeat_sp.py:28-193."""
     steps = ar_video_steps(k.shape[1], mini_batch_size, update_length, update_every, num_repeat)
     out, ws, _ = run_program(
-        w0, w1, w2, q, k, v, lr0 * w_scale, lr1 * w_scale, lr2 * w_scale, steps, num=num,
+        w0, w1, w2, q, k, v, lr0, lr1, lr2, steps, num=num, w_scale=w_scale,
         ns_coeffs=ns_coeff_table("classic", num_moun_iters) if use_moun else None,
         momentum=fw_momentum if use_momentum else None, weight_norm=weight_norm,
         cast_lr_operand=False)
@@ -478,7 +482,7 @@ def ar_fast_weight_swish_glu_weight_norm_mini_batch_inference(w0, w1, w2, q, k, 
     steps = [Step(UPDATE, 0, mb) for _ in range(num_repeat)] if do_update else []
     steps.append(Step(APPLY, 0, q.shape[1]))
     out, ws, _ = run_program(
-        w0, w1, w2, q, k, v, lr0 * w_scale, lr1 * w_scale, lr2 * w_scale, steps, num=num,
+        w0, w1, w2, q, k, v, lr0, lr1, lr2, steps, num=num, w_scale=w_scale,
         ns_coeffs=ns_coeff_table("classic", num_moun_iters) if use_moun else None,
         weight_norm=weight_norm, cast_lr_operand=False)
     return (out,) + tuple(ws)
@@ -500,7 +504,7 @@ def ar_fast_weight_swish_glu_weight_norm_mini_batch_inference_with_momentum(
         state = ((dw0_momentum, dw1_momentum, dw2_momentum) if dw0_momentum is not None
                  else (torch.zeros_like(w0), torch.zeros_like(w1), torch.zeros_like(w2)))
     out, ws, ms = run_program(
-        w0, w1, w2, q, k, v, lr0 * w_scale, lr1 * w_scale, lr2 * w_scale, steps, num=num,
+        w0, w1, w2, q, k, v, lr0, lr1, lr2, steps, num=num, w_scale=w_scale,
         ns_coeffs=ns_coeff_table("classic", num_moun_iters) if use_moun else None,
         momentum=fw_momentum if use_momentum else None, weight_norm=weight_norm,
         cast_lr_operand=False, momentum_state=state)
