@@ -134,7 +134,8 @@ int lact_newton_schulz_backward(int32_t n, int32_t rows, int32_t cols, const flo
  * until the process ends; the call allocates nothing.  Shapes whose lact_newton_schulz_workspace_bytes exceed it are
  * refused (return value < 0, message in lact_last_error).  Every call on a GPU uses that GPU's one array: calls that
  * overlap on one GPU (two streams, two threads) race; calls on one stream are ordered by the stream.  Same kernels
- * and same results, bit for bit, as lact_newton_schulz. */
+ * and same results, bit for bit, as lact_newton_schulz.  The first call on a device looks up the array's address and
+ * sets kernel attributes: make one call outside any graph capture before capturing one. */
 #define LACT_NS_STATIC_WORKSPACE_BYTES (32u << 20)
 size_t lact_newton_schulz_static_capacity(void);
 int lact_newton_schulz_static(int32_t n, int32_t rows, int32_t cols, const float* g, float* out, int32_t steps,

@@ -58,3 +58,46 @@ def test_static_workspace_newton_schulz_matches_the_workspace_entry_point():
     rc = L.lact_newton_schulz_static(n, rows, cols, _ptr(g), _ptr(g), 5, _coeffs(O.NS5_COEFFS), 0,
                                      ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
     assert rc != 0 and b"static workspace holds" in L.lact_last_error()
+
+
+def test_static_entry_point_allocates_nothing_and_replays_from_a_graph():
+    """What the entry point exists for: after one warm-up call (which looks up the array's address and sets kernel
+    attributes -- do that outside a capture), a call changes neither the device's free memory nor torch's allocator
+    counters, and the call captured into a HIP graph replays to the same bits, several times, with eager work between
+    the replays."""
+    L = _lib.lib()
+    gen = torch.Generator().manual_seed(29)
+    n, rows, cols, co, mode = 3, 192, 384, O.ns_coeff_table("llm", 5), 0
+    G = torch.randn(n, rows, cols, generator=gen)
+    got, want = _both(L, G, co, mode)                       # warm-up of both entry points
+    assert torch.equal(got, want)
+    g = G.to(DEV).contiguous()
+    out = torch.full_like(g, float("nan"))
+    arr = _coeffs(co)
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    alloc0, reserved0 = torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _lib.check(L.lact_newton_schulz_static(n, rows, cols, _ptr(g), _ptr(out), len(co), arr, mode, stream))
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0 and torch.cuda.memory_allocated() == alloc0 and torch.cuda.memory_reserved() == reserved0
+    assert torch.equal(out, want)
+    # captured: the call records kernels only (no allocation, no memset)
+    out_g = torch.full_like(g, float("nan"))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            s = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            _lib.check(L.lact_newton_schulz_static(n, rows, cols, _ptr(g), _ptr(out_g), len(co), arr, mode, s))
+    torch.cuda.current_stream().wait_stream(side)
+    for i in range(3):
+        out_g.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, want), i
+        # eager work of the program's own between the replays, on the same array
+        got2, want2 = _both(L, torch.randn(2, 64, 128, generator=gen), O.ns_coeff_table("classic", 3), 0)
+        assert torch.equal(got2, want2)
