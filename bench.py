@@ -111,6 +111,9 @@ def main():
     ap.add_argument("--no-overlap", action="store_true",
                     help="keep the apply steps on the caller's stream (LACT_OPT_STREAM_OVERLAP off): kernels then run "
                          "one at a time and their durations are those of the kernel alone; used for profiles")
+    ap.add_argument("--persistent-tiles", type=int, default=None,
+                    help="LACT_OPT_PERSISTENT_TILES mask (bit 0 apply, 1 update, 2 apply backward hidden stage; default: the "
+                         "library's, all on); 0 runs the one-tile-per-block kernels for comparison")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (three times): the known-size kernel that scales the "
                          "FETCH_SIZE / WRITE_SIZE counters of a `rocprofv3 --pmc` run of this command")
@@ -241,6 +244,8 @@ def main():
 
     if args.no_overlap:
         _lib.lib().lact_set_option(_lib.OPT_STREAM_OVERLAP, 0)
+    if args.persistent_tiles is not None:
+        _lib.lib().lact_set_option(_lib.OPT_PERSISTENT_TILES, args.persistent_tiles)
     for _ in range(args.warmup):
         step()
     # `repeats` timed regions of exactly `steps` steps each, every one bracketed by a device synchronisation; the

@@ -176,7 +176,7 @@ int lact_layer_post_backward(int32_t act_dtype, int32_t B, int32_t L, int32_t H,
                              const void* dy, void* d_o, void* dgate_raw, float* dw_part, void* stream);
 
 /* Execution options (process-wide; no counterpart in the reference, where PyTorch enqueues the whole layer on one
- * stream as separate kernels).  Both are on by default and change no result bit.
+ * stream as separate kernels).  The switches are on by default and change no result bit.
  *   LACT_OPT_STREAM_OVERLAP: the apply steps of a program do not depend on the update chain that runs beside
  *     them, and nothing in a call waits for dk, dv or the learning-rate gradients of an update; lact_forward /
  *     lact_backward enqueue them on two library-owned streams (default priority, per device, created on first
@@ -189,8 +189,13 @@ int lact_layer_post_backward(int32_t act_dtype, int32_t B, int32_t L, int32_t H,
  *     before it gives up (value <= 0 restores the default, a fraction of a second).  A block that gives up raises
  *     an error word and goes on, so every kernel always ends; the step's results (weights, outputs that depend on
  *     them, gradients) are then NaN.  Meant for tests of that path.
+ *   LACT_OPT_PERSISTENT_TILES: the hidden-stage kernels (bf16, d a multiple of 64) run as one block per compute unit
+ *     that walks its share of the tiles, the copy waves running ahead into the next tile and doing the previous
+ *     tile's epilogue beside the matrix waves; otherwise one tile per block.  Same arithmetic, same bits.  The value
+ *     is a mask: bit 0 the apply's hidden stage, bit 1 the update's, bit 2 the apply backward's (default: 5; the
+ *     update's hidden stage, whose epilogue writes up to eight arrays, measured faster as one tile per block).
  * Returns the previous value (0 / 1, or the previous limit), or -1 for an unknown option. */
-enum { LACT_OPT_STREAM_OVERLAP = 0, LACT_OPT_FUSED_NEWTON_SCHULZ = 1, LACT_OPT_NS_BARRIER_SPIN_LIMIT = 2 };
+enum { LACT_OPT_STREAM_OVERLAP = 0, LACT_OPT_FUSED_NEWTON_SCHULZ = 1, LACT_OPT_NS_BARRIER_SPIN_LIMIT = 2, LACT_OPT_PERSISTENT_TILES = 3 };
 int lact_set_option(int32_t option, int32_t value);
 
 /* Errors that only the device notices.  A block of the fused Newton-Schulz kernel that gives up at a barrier (see

@@ -16,6 +16,7 @@
 
 #include "gemm_dma_kernels.h"
 #include "ns_fused.h"
+#include "gemm_persist.h"
 #include "gemm_kernels.h"
 #include "state_kernels.h"
 #include "layer_kernels.h"
@@ -160,6 +161,8 @@ static __device__ unsigned g_async_errors;
 namespace {
 bool g_overlap = true;
 bool g_fused_ns = true;
+int g_persist = 5;          // hidden-stage kernels on the persistent engine (LACT_OPT_PERSISTENT_TILES): bit 0 apply, 1 update, 2 apply backward
+                            // (the update's eight-output epilogue is faster staged through the whole ring by all eight waves: off by default)
 long long g_ns_spin_limit = NS_FUSED_SPIN_LIMIT;   // barrier wait bound of the fused Newton-Schulz kernels (lact_set_option)
 std::mutex g_enqueue_mutex;   // one program is enqueued at a time (the side-stream context is shared)
 SideCtx* side_ctx() {
@@ -698,6 +701,18 @@ struct Runner {
       LACT_BIG_LDS(k_apply_bwd_hidden_dma<TS_SQ>, SM3);
       LACT_BIG_LDS(k_update_bwd_hidden_dma<TS_BWD>, SM6);
       LACT_BIG_LDS(k_update_bwd_hidden_kept_dma<TS_SQ>, SM3);
+      if (which <= 2 && ((g_persist >> which) & 1) && side && side->cus > 0) {
+        HiddenPersistParams hq;
+        hq.h = hp; hq.map = m3;
+        const dim3 gp(persist_grid(m3.grid(), side->cus));
+        LACT_BIG_LDS(k_hidden_persist<ApplyHiddenPolicy>, PersistLds<ApplyHiddenPolicy>::BYTES);
+        LACT_BIG_LDS(k_hidden_persist<UpdateHiddenPolicy>, PersistLds<UpdateHiddenPolicy>::BYTES);
+        LACT_BIG_LDS(k_hidden_persist<ApplyBwdHiddenPolicy>, PersistLds<ApplyBwdHiddenPolicy>::BYTES);
+        if (which == 0) LACT_LAUNCH_SMEM("k_hidden_persist<apply>", "apply_hidden", 4.0 * f, (k_hidden_persist<ApplyHiddenPolicy>), gp, dim3(DMA_THREADS), PersistLds<ApplyHiddenPolicy>::BYTES, s, hq);
+        if (which == 1) LACT_LAUNCH_SMEM("k_hidden_persist<update>", "update_hidden", 6.0 * f, (k_hidden_persist<UpdateHiddenPolicy>), gp, dim3(DMA_THREADS), PersistLds<UpdateHiddenPolicy>::BYTES, s, hq);
+        if (which == 2) LACT_LAUNCH_SMEM("k_hidden_persist<apply_bwd>", "apply_bwd_hidden", 6.0 * f, (k_hidden_persist<ApplyBwdHiddenPolicy>), gp, dim3(DMA_THREADS), PersistLds<ApplyBwdHiddenPolicy>::BYTES, s, hq);
+        return;
+      }
       if (which == 0) LACT_LAUNCH_SMEM("k_apply_hidden_dma", "apply_hidden", 4.0 * f, (k_apply_hidden_dma<TS_SQ>), g3, dim3(DMA_THREADS), SM3, s, q);
       if (which == 1) LACT_LAUNCH_SMEM("k_update_hidden_dma", "update_hidden", 6.0 * f, (k_update_hidden_dma<TS_SQ>), g3, dim3(DMA_THREADS), SM3, s, q);
       if (which == 2) LACT_LAUNCH_SMEM("k_apply_bwd_hidden_dma", "apply_bwd_hidden", 6.0 * f, (k_apply_bwd_hidden_dma<TS_SQ>), g3, dim3(DMA_THREADS), SM3, s, q);
@@ -1863,6 +1878,11 @@ int lact_set_option(int32_t option, int32_t value) {
     g_ns_spin_limit = value > 0 ? value : NS_FUSED_SPIN_LIMIT;
     return (int)std::min<long long>(was, 0x7fffffff);
   }
+  if (option == LACT_OPT_PERSISTENT_TILES) {
+    const int was = g_persist;
+    g_persist = value;
+    return was;
+  }
   bool* flag = option == LACT_OPT_STREAM_OVERLAP ? &g_overlap : (option == LACT_OPT_FUSED_NEWTON_SCHULZ ? &g_fused_ns : nullptr);
   if (!flag) return fail("lact_set_option: unknown option");
   const int was = *flag ? 1 : 0;
@@ -2023,6 +2043,17 @@ int lact_mfma_calibration(int32_t blocks, int32_t iters, float* out, void* strea
   LACT_CHECK_LAUNCH();
   return 0;
 }
+
+#ifdef LACT_PERSIST_TS
+int lact_debug_timestamps(void* host, size_t bytes) {   // timing experiments only
+  (void)hipDeviceSynchronize();
+  return hipMemcpyFromSymbol(host, HIP_SYMBOL(g_pts), std::min(bytes, sizeof(g_pts)), 0, hipMemcpyDeviceToHost) == hipSuccess ? 0 : -1;
+}
+int lact_debug_timestamps_clear(void) {
+  static std::vector<unsigned> z(sizeof(g_pts) / 4, 0);
+  return hipMemcpyToSymbol(HIP_SYMBOL(g_pts), z.data(), sizeof(g_pts), 0, hipMemcpyHostToDevice) == hipSuccess ? 0 : -1;
+}
+#endif
 
 int lact_profile_enable(int on) {
   g_prof.clear();

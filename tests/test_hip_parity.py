@@ -1122,6 +1122,45 @@ def test_stream_overlap_is_bit_identical(prenorm):
     assert torch.equal(on[0][0], on[2][0]) and all(torch.equal(on[0][1][n], on[2][1][n]) for n in on[0][1])
 
 
+@pytest.mark.parametrize("b,L,d,dh,C,muon", [
+    (2, 3 * 128 + 40, 128, 128, 128, False),      # ragged last token tile, one hidden tile
+    (3, 2 * 300 + 50, 64, 192, 300, True),        # dh = 128 + 64: a half-valid hidden tile; chunk not a multiple of 128
+    (5, 3 * 256, 128, 256, 256, True),            # batch not a multiple of 8 (tile map by rows of tiles)
+    (16, 2 * 1024 + 7, 384, 384, 1024, True),     # config-1 head shape, several tiles per block
+    (1, 2 * 64, 64, 64, 64, False)])              # fewer tiles than compute units, one K-step per phase
+def test_persistent_tiles_are_bit_identical(b, L, d, dh, C, muon):
+    """The hidden-stage kernels as persistent blocks (copy waves running ahead across tiles and doing the previous
+    tile's epilogue beside the matrix waves) against one tile per block: the same arithmetic in the same order, so the
+    same bits in the output and in every gradient."""
+    say("persistent tiles on/off", b, L, d, dh, C, muon)
+    from lact_amd import _lib
+    inp = problem(b, L, d, dh, seed=55, act=torch.bfloat16)
+    go = torch.randn(b, L, d, generator=torch.Generator().manual_seed(8)).bfloat16().to(DEV)
+
+    def run():
+        res = []
+        for _ in range(2):
+            t = clone_to(inp, DEV)
+            out = T.block_causal_lact_swiglu(*args9(t), C, muon, t["momentum"])
+            res.append((out, grads_of(out, t, go)))
+        torch.cuda.synchronize()
+        return res
+    L_ = _lib.lib()
+    prev = L_.lact_set_option(_lib.OPT_PERSISTENT_TILES, 7)      # all three hidden-stage kernels persistent
+    try:
+        on = run()
+        L_.lact_set_option(_lib.OPT_PERSISTENT_TILES, 0)
+        off = run()
+    finally:
+        L_.lact_set_option(_lib.OPT_PERSISTENT_TILES, prev)
+    for (o1, g1), (o0, g0) in zip(on, off):
+        assert torch.isfinite(o1.float()).all()
+        assert torch.equal(o1, o0)
+        for n in g0:
+            assert torch.equal(g1[n], g0[n]), (n, O.rel_l2(g1[n], g0[n]))
+    assert all(torch.equal(on[0][1][n], on[1][1][n]) for n in on[0][1])
+
+
 @pytest.mark.parametrize("chunks", [2, 3])
 @pytest.mark.parametrize("b,d,dh", [(5, 384, 192), (2, 384, 384), (4, 384, 384), (3, 256, 128),
                                     (2, 768, 1536)])   # the video model's head: 32 blocks per matrix, a whole XCD per group
