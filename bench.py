@@ -59,6 +59,9 @@ def _library_label(profile_name):
     if m:
         epi = {"0": "store", "1": "axpby", "2": "axpby_dual"}[m.group(3)]
         return f"k_row_gemm_dma<{m.group(1)},{m.group(2)},{epi},{'Bks' if m.group(4) == 'true' else 'Bkc'}>"
+    m = re.match(r"k_hidden_persist<(Apply|Update|ApplyBwd)HiddenPolicy>", n)
+    if m:
+        return f"k_hidden_persist<{ {'Apply': 'apply', 'Update': 'update', 'ApplyBwd': 'apply_bwd'}[m.group(1)] }>"
     m = re.match(r"(k_token_reduce(?:_rows)?_dma)<(\d+x\d+)>", n)
     if m:
         return f"{m.group(1)}<{m.group(2)}>"
@@ -113,7 +116,7 @@ def main():
                          "one at a time and their durations are those of the kernel alone; used for profiles")
     ap.add_argument("--persistent-tiles", type=int, default=None,
                     help="LACT_OPT_PERSISTENT_TILES mask (bit 0 apply, 1 update, 2 apply backward hidden stage; default: the "
-                         "library's, all on); 0 runs the one-tile-per-block kernels for comparison")
+                         "library's, 1); 0 runs the one-tile-per-block kernels for comparison")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (three times): the known-size kernel that scales the "
                          "FETCH_SIZE / WRITE_SIZE counters of a `rocprofv3 --pmc` run of this command")

@@ -190,10 +190,12 @@ int lact_layer_post_backward(int32_t act_dtype, int32_t B, int32_t L, int32_t H,
  *     an error word and goes on, so every kernel always ends; the step's results (weights, outputs that depend on
  *     them, gradients) are then NaN.  Meant for tests of that path.
  *   LACT_OPT_PERSISTENT_TILES: the hidden-stage kernels (bf16, d a multiple of 64) run as one block per compute unit
- *     that walks its share of the tiles, the copy waves running ahead into the next tile and doing the previous
- *     tile's epilogue beside the matrix waves; otherwise one tile per block.  Same arithmetic, same bits.  The value
- *     is a mask: bit 0 the apply's hidden stage, bit 1 the update's, bit 2 the apply backward's (default: 5; the
- *     update's hidden stage, whose epilogue writes up to eight arrays, measured faster as one tile per block).
+ *     that walks its share of the tiles, the copy waves running ahead into the next tile while the matrix waves run
+ *     the previous tile's epilogue; otherwise one tile per block.  Same arithmetic, same bits.  The value is a mask:
+ *     bit 0 the apply's hidden stage, bit 1 the update's, bit 2 the apply backward's.  Default: 1.  The update's
+ *     hidden stage, whose epilogue writes up to eight arrays, measured slower this way; the apply backward's measured
+ *     2 % faster as a kernel but runs beside other kernels on a second stream, where a launch that holds every
+ *     compute unit until its last tile costs the step more than it saves.
  * Returns the previous value (0 / 1, or the previous limit), or -1 for an unknown option. */
 enum { LACT_OPT_STREAM_OVERLAP = 0, LACT_OPT_FUSED_NEWTON_SCHULZ = 1, LACT_OPT_NS_BARRIER_SPIN_LIMIT = 2, LACT_OPT_PERSISTENT_TILES = 3 };
 int lact_set_option(int32_t option, int32_t value);

@@ -3,79 +3,59 @@
 //   matrix waves  (0-3): fragments from the LDS ring, MFMAs, and at the end of a tile its epilogue, straight from the
 //                        accumulators;
 //   service waves (4-7): the asynchronous global -> LDS copies of the ring, in one flat sequence over all phases of all
-//                        tiles of the block: while the matrix waves run a tile's epilogue, the next tile's first
-//                        stages are already landing (three stages ahead, the whole ring).
+//                        tiles of the block: while the matrix waves run a tile's epilogue, the next tile's first two
+//                        stages are already landing.
 //
-// Why this pays: the main loops of these kernels run at the rate a compute unit can copy operands into its LDS (about
-// 1 us per 48 KiB K-step against 0.5 us of matrix work, measured with the epilogue switched off), so the matrix
-// waves have slack.  With one tile per block the ring's fill, the epilogue and the dispatcher's lock-step rounds were
-// paid in line, copy engine idle; here the epilogue costs only what it exceeds the ring's three stages of run-ahead.
-// Measured and rejected on the way: the epilogue on the copy waves, fed through LDS (hand-over of the rounded
-// accumulators), to run it "beside" the matrix work -- a wave stalls in order while its copy instructions wait for the
-// address queue, so a copy wave cannot compute during the copies it issues, and every epilogue instruction it
-// executes delays the next stage: apply 37.3 us per launch against 37.4 for one tile per block, update 150 against 92.
+// Why this pays: with one tile per block the ring's fill, the epilogue and the dispatcher's lock-step rounds are paid in
+// line, copy engine idle; here the next tile's fill hides behind the epilogue.  What it does not change is the main
+// loop itself: a 48 KiB K-step takes 0.75-1 us to copy against 0.43 us of matrix work (measured with the matrix work and
+// the epilogue switched off: the copies alone take 18-20 us of a 33 us launch at 18 K-steps per block).
+//
+// Measured and rejected on the way:
+//   * the epilogue on the copy waves, fed through LDS (hand-over of the rounded accumulators), to run it "beside" the
+//     matrix work -- a wave stalls in order while its copy instructions wait for the address queue, so a copy wave
+//     cannot compute during the copies it issues, and every epilogue instruction it executes delays the next stage:
+//     apply 37.3 us per launch against 37.4 for one tile per block, update 150 against 92;
+//   * the matrix waves touching every 128-byte line of the next tile's token rows a tile ahead (one 4-byte asynchronous
+//     copy per line into an LDS area nobody reads), so that the rows are in the L2 when their copies run: apply 36.6 us
+//     against 34.0, apply backward 65.5 against 59.2 -- the touches cost a stage's worth of address processing per tile
+//     and the copies behind them are no faster;
+//   * all hidden tiles of a token tile on one block, back to back, so that the token rows come from HBM once and from
+//     the L2 twice: apply 36.6 us against 33.4, apply backward 62.5 against 58.2 (three blocks that fetch the same rows
+//     at the same moment share one HBM fetch just as well).
 //
 // Epilogue stores.  A lane owns 4 consecutive columns of 32 different rows per 32 x 32 fragment; stored straight from
-// the accumulators that is 32 cache lines per instruction.  Every matrix wave has a 4 KiB window of LDS of its own
-// (behind the ring: 3 x 48 KiB + 16 KiB = the whole 160 KiB): it writes a fragment of results there as [32 rows][64
-// bytes], reads it back row-wise (4 lanes x 16 bytes per row) and stores 64-byte row segments.  The window is private
-// to the wave, LDS operations of a wave execute in order: no barrier is involved.
+// the accumulators that is 32 cache lines per instruction.  The ring slot of the tile's last K-step is free once every
+// matrix wave is past its last fetch (one block barrier): each matrix wave stages up to six fragments of results there
+// as [32 rows][64 bytes], reads them back row-wise (4 lanes x 16 bytes per row) and stores 64-byte row segments, all
+// reads of a group before its stores.  The part of the slot a wave uses is its own and the LDS operations of a wave
+// execute in order: no further barrier.  The copy waves refill that slot only after the next tile's first barrier.
 #pragma once
 #include <algorithm>
 
 #include "gemm_dma_kernels.h"
 
-// Optional in-kernel timestamps (timing experiments build with -DLACT_PERSIST_TS; nothing in the library otherwise).
-#ifdef LACT_PERSIST_TS
-// Records go to LDS while the kernel runs (no global store perturbs the copy queue) and are copied out at the end.
-static __device__ unsigned g_pts[256 * 2 * 128 * 2];
-#define LACT_PTS_LDS_BYTES (2 * 128 * 8)
-__device__ __forceinline__ unsigned lact_now() {
-  unsigned long long t;
-  asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t)::"memory");
-  return (unsigned)t;
-}
-#define LACT_PTS(role, n, tag)                                                                       \
-  do {                                                                                               \
-    if ((threadIdx.x & 63) == 0 && ((threadIdx.x >> 6) & 3) == 0 && (n) < 128) {                     \
-      unsigned* e_ = reinterpret_cast<unsigned*>(lact_pts_lds) + ((role) * 128 + (n)) * 2;           \
-      e_[0] = (tag);                                                                                 \
-      e_[1] = lact_now();                                                                            \
-      ++(n);                                                                                         \
-    }                                                                                                \
-  } while (0)
-#define LACT_PTS_FLUSH(role, n)                                                                      \
-  do {                                                                                               \
-    if ((threadIdx.x & 63) == 0 && ((threadIdx.x >> 6) & 3) == 0 && blockIdx.x < 256) {              \
-      const unsigned* e_ = reinterpret_cast<const unsigned*>(lact_pts_lds) + (role) * 256;           \
-      for (int i_ = 0; i_ < 2 * (n); ++i_) g_pts[((size_t)blockIdx.x * 2 + (role)) * 256 + i_] = e_[i_]; \
-    }                                                                                                \
-  } while (0)
-#else
-#define LACT_PTS_LDS_BYTES 0
-#define LACT_PTS(role, n, tag) do { (void)(n); } while (0)
-#define LACT_PTS_FLUSH(role, n) do { (void)(n); } while (0)
-#endif
-
 namespace lact {
 
 constexpr int PS_STAGES = 3;
 
-// s_waitcnt vmcnt(n) for a wave-uniform run-time n (clamped to the counter's range; a smaller n only waits longer).
-// The immediate must be a constant: a balanced tree of scalar branches picks it (six compares).
-template <int LO, int HI>
-__device__ __forceinline__ void wait_vmcnt_tree(int n) {
-  if constexpr (LO == HI) {
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LO) : "memory");
-  } else {
-    constexpr int MID = (LO + HI) / 2;
-    if (n <= MID) wait_vmcnt_tree<LO, MID>(n);
-    else wait_vmcnt_tree<MID + 1, HI>(n);
-  }
-}
+// s_waitcnt vmcnt(n) for a wave-uniform run-time n.  The immediate must be a constant, so n is rounded DOWN to a
+// multiple of four (a smaller count only waits longer; the copy waves issue copies in fours) and a short chain of scalar
+// branches picks it.  The chain is on the copy waves' critical path once per K-step: a wave issues an instruction
+// every four or five cycles at best and a taken branch costs a few times that, so a 64-leaf tree here cost 1-2 us per
+// launch.
 __device__ __forceinline__ void wait_vmcnt_dyn(int n) {
   n = __builtin_amdgcn_readfirstlane(n);
-  wait_vmcnt_tree<0, 63>(n < 0 ? 0 : (n > 63 ? 63 : n));
+  if (n >= 12) {
+    if (n >= 24) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+    else if (n >= 20) asm volatile("s_waitcnt vmcnt(20)" ::: "memory");
+    else if (n >= 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+  } else {
+    if (n >= 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else if (n >= 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
 }
 
 // ---- tile list of a block: tiles b, b + G, b + 2 G, ... of the launch's tile map (G = grid, a multiple of 8: all of a
@@ -133,7 +113,7 @@ __device__ __forceinline__ void frag_store(const uint4 (&v)[2], uint16_t* out, i
 
 // ---- service side: the copy cursor ------------------------------------------------------------------------------------
 // Issues the ring's stages in order over the phases of a tile and on into the next tile's, and keeps the count of
-// vector-memory operations this wave has issued (copies here, stores by the epilogue through `ops`).
+// vector-memory operations this wave has issued, from which the wait for a stage derives its vmcnt.
 template <class TS, int NB, int NPH>
 struct CopyCursor {
   using SM = DmaSmem<TS, NB, PS_STAGES>;
@@ -169,14 +149,14 @@ struct CopyCursor {
       }
     ckt = 0;
   }
-  // next(ph, cursor) fills the phases of the following tile (and may issue copies of its own, adding them to `ops`);
-  // returns false when there is no further tile
+  // next(ph, ops) fills the phases of the following tile; returns false when there is no further tile
   template <class Next>
   __device__ __forceinline__ void advance(Next& next) {
-    for (;;) {
+    valid = false;
+    for (int tries = 0; tries <= NPH; ++tries) {   // a tile has at least one phase with K-steps
       ++cp;
       if (cp >= NPH) {
-        if (!next(ph, ops)) { valid = false; return; }
+        if (!next(ph, ops)) return;
         cp = 0;
       }
       select_phase();
@@ -390,14 +370,11 @@ struct UpdateHiddenPolicy {
 };
 
 // ---- the kernel --------------------------------------------------------------------------------------------------------
-#ifndef LACT_PERSIST_EXP
-#define LACT_PERSIST_EXP 0
-#endif
 template <class POL>
 struct PersistLds {
   using SM = DmaSmem<typename POL::TS, POL::NB, PS_STAGES>;
   static constexpr int RING = SM::BYTES;
-  static constexpr int BYTES = RING + LACT_PTS_LDS_BYTES;
+  static constexpr int BYTES = RING;
   static_assert(SM::STAGE >= WINDOW_BYTES, "the epilogue window is the ring slot of a tile's last K-step");
 };
 
@@ -425,8 +402,6 @@ __global__ __launch_bounds__(DMA_THREADS) void k_hidden_persist(const HiddenPers
   using L = PersistLds<POL>;
   static_assert(TS::BM == 128 && TS::BN == 128 && TS::WM == 64 && TS::WN == 64, "64 x 64 per wave");
   const HiddenParams& p = pp.h;
-  char* lact_pts_lds = smem + L::RING;
-  (void)lact_pts_lds;
   const bool service = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) >= 4;
   // K-steps of a tile (the same for every tile of the launch)
   int nk_tile;
@@ -438,7 +413,6 @@ __global__ __launch_bounds__(DMA_THREADS) void k_hidden_persist(const HiddenPers
     for (int i = 0; i < POL::NPH; ++i) nk_tile += ph0[i].K / DMA_BK;
   }
   if (nk_tile <= 0) return;
-  int nts = 0;
 
   if (service) {
     // ------------------------------------------------------------------------------------------ service waves
@@ -453,7 +427,6 @@ __global__ __launch_bounds__(DMA_THREADS) void k_hidden_persist(const HiddenPers
     int g = 0;               // K-steps consumed so far (all tiles)
     for (int i = 0; i < PS_STAGES - 1 && cur.valid; ++i) cur.issue_stage(next_tile);
     int lin;
-    LACT_PTS(1, nts, 1);
     while (walk.take(lin)) {
       int bx, by, z;
       if (!pp.map.locate(lin, bx, by, z)) continue;
@@ -466,9 +439,7 @@ __global__ __launch_bounds__(DMA_THREADS) void k_hidden_persist(const HiddenPers
       // the matrix waves' end-of-loop barrier.  The slot of the tile's last K-step is their epilogue window until they
       // reach the next tile's first barrier: two stages of the next tile are in flight meanwhile.
       __syncthreads();
-      LACT_PTS(1, nts, 2);
     }
-    LACT_PTS_FLUSH(1, nts);
   } else {
     // ------------------------------------------------------------------------------------------- matrix waves
     using Pipe = DmaPipe<TS, POL::NB, POL::NPH, PS_STAGES>;
@@ -483,24 +454,16 @@ __global__ __launch_bounds__(DMA_THREADS) void k_hidden_persist(const HiddenPers
     while (walk.take(lin)) {
       int bx, by, z;
       if (!pp.map.locate(lin, bx, by, z)) continue;
-      LACT_PTS(0, nts, 11);
       zero_acc<TS>(a02[0]);
       zero_acc<TS>(a02[1]);
       if (POL::NACC > 2) zero_acc<TS>(a1[0]);
       POL::mma(pipe, p, step, a02, a1);
-      LACT_PTS(0, nts, 12);
-      if (LACT_PERSIST_EXP == 4) {
-        asm volatile("" ::"v"(a02[0][0][0]), "v"(a02[1][1][1]), "v"(a02[0][1][0]), "v"(a02[1][0][1]), "v"(a02[0][0][1]), "v"(a02[0][1][1]), "v"(a02[1][0][0]), "v"(a02[1][1][0]));
-        continue;
-      }
       // Window: the slot of the K-step just finished.  Every matrix wave read fragments from all of it, so all of them
       // must be past their last fetch before any of them writes there: one barrier (the copy waves join it).
       __syncthreads();
       f.init(smem + ((step - 1) % PS_STAGES) * L::SM::STAGE, bx * TS::BM, by * TS::BN, z, p.T, p.dh);
       POL::epilogue(p, f, a02, a1);
-      LACT_PTS(0, nts, 13);
     }
-    LACT_PTS_FLUSH(0, nts);
   }
 }
 

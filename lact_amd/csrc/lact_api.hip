@@ -161,7 +161,7 @@ static __device__ unsigned g_async_errors;
 namespace {
 bool g_overlap = true;
 bool g_fused_ns = true;
-int g_persist = 5;          // hidden-stage kernels on the persistent engine (LACT_OPT_PERSISTENT_TILES): bit 0 apply, 1 update, 2 apply backward
+int g_persist = 1;          // hidden-stage kernels on the persistent engine (LACT_OPT_PERSISTENT_TILES): bit 0 apply, 1 update, 2 apply backward
                             // (the update's eight-output epilogue is faster staged through the whole ring by all eight waves: off by default)
 long long g_ns_spin_limit = NS_FUSED_SPIN_LIMIT;   // barrier wait bound of the fused Newton-Schulz kernels (lact_set_option)
 std::mutex g_enqueue_mutex;   // one program is enqueued at a time (the side-stream context is shared)
@@ -2043,17 +2043,6 @@ int lact_mfma_calibration(int32_t blocks, int32_t iters, float* out, void* strea
   LACT_CHECK_LAUNCH();
   return 0;
 }
-
-#ifdef LACT_PERSIST_TS
-int lact_debug_timestamps(void* host, size_t bytes) {   // timing experiments only
-  (void)hipDeviceSynchronize();
-  return hipMemcpyFromSymbol(host, HIP_SYMBOL(g_pts), std::min(bytes, sizeof(g_pts)), 0, hipMemcpyDeviceToHost) == hipSuccess ? 0 : -1;
-}
-int lact_debug_timestamps_clear(void) {
-  static std::vector<unsigned> z(sizeof(g_pts) / 4, 0);
-  return hipMemcpyToSymbol(HIP_SYMBOL(g_pts), z.data(), sizeof(g_pts), 0, hipMemcpyHostToDevice) == hipSuccess ? 0 : -1;
-}
-#endif
 
 int lact_profile_enable(int on) {
   g_prof.clear();
