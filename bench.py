@@ -117,6 +117,9 @@ def main():
     ap.add_argument("--persistent-tiles", type=int, default=None,
                     help="LACT_OPT_PERSISTENT_TILES mask (bit 0 apply, 1 update, 2 apply backward hidden stage; default: the "
                          "library's, 1); 0 runs the one-tile-per-block kernels for comparison")
+    ap.add_argument("--keep-preactivations", type=int, default=None,
+                    help="LACT_OPT_KEEP_PREACTIVATIONS: 0 the update's backward recomputes its hidden stage, 1 the forward "
+                         "keeps the rounded pre-activations and lr-scaled operands (default: the library's choice by shape)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (three times): the known-size kernel that scales the "
                          "FETCH_SIZE / WRITE_SIZE counters of a `rocprofv3 --pmc` run of this command")
@@ -249,6 +252,8 @@ def main():
         _lib.lib().lact_set_option(_lib.OPT_STREAM_OVERLAP, 0)
     if args.persistent_tiles is not None:
         _lib.lib().lact_set_option(_lib.OPT_PERSISTENT_TILES, args.persistent_tiles)
+    if args.keep_preactivations is not None:
+        _lib.lib().lact_set_option(_lib.OPT_KEEP_PREACTIVATIONS, args.keep_preactivations)
     for _ in range(args.warmup):
         step()
     # `repeats` timed regions of exactly `steps` steps each, every one bracketed by a device synchronisation; the

@@ -196,8 +196,13 @@ int lact_layer_post_backward(int32_t act_dtype, int32_t B, int32_t L, int32_t H,
  *     hidden stage, whose epilogue writes up to eight arrays, measured slower this way; the apply backward's measured
  *     2 % faster as a kernel but runs beside other kernels on a second stream, where a launch that holds every
  *     compute unit until its last tile costs the step more than it saves.
+ *   LACT_OPT_KEEP_PREACTIVATIONS: 1: the update's forward keeps its rounded pre-activations and lr-scaled operands
+ *     for the backward (bf16, d and dh multiples of 64), 0: the backward recomputes them, -1 (default): by shape
+ *     (kept when d > 128).  Same bits either way, except the learning-rate gradients (fp32 sums over tiles of another
+ *     width: 1e-7).  Read when a call is planned: set it before the
+ *     forward and leave it until that forward's backward has been enqueued (the two must agree on what was saved).
  * Returns the previous value (0 / 1, or the previous limit), or -1 for an unknown option. */
-enum { LACT_OPT_STREAM_OVERLAP = 0, LACT_OPT_FUSED_NEWTON_SCHULZ = 1, LACT_OPT_NS_BARRIER_SPIN_LIMIT = 2, LACT_OPT_PERSISTENT_TILES = 3 };
+enum { LACT_OPT_STREAM_OVERLAP = 0, LACT_OPT_FUSED_NEWTON_SCHULZ = 1, LACT_OPT_NS_BARRIER_SPIN_LIMIT = 2, LACT_OPT_PERSISTENT_TILES = 3, LACT_OPT_KEEP_PREACTIVATIONS = 4 };
 int lact_set_option(int32_t option, int32_t value);
 
 /* Errors that only the device notices.  A block of the fused Newton-Schulz kernel that gives up at a barrier (see

@@ -34,7 +34,7 @@ class Desc(Structure):
     ]
 
 
-OPT_STREAM_OVERLAP, OPT_FUSED_NEWTON_SCHULZ, OPT_NS_BARRIER_SPIN_LIMIT, OPT_PERSISTENT_TILES = 0, 1, 2, 3
+OPT_STREAM_OVERLAP, OPT_FUSED_NEWTON_SCHULZ, OPT_NS_BARRIER_SPIN_LIMIT, OPT_PERSISTENT_TILES, OPT_KEEP_PREACTIVATIONS = 0, 1, 2, 3, 4
 EXPORTS = ("lact_last_error", "lact_version", "lact_query_sizes", "lact_forward", "lact_forward_from_state", "lact_backward",
            "lact_newton_schulz_workspace_bytes", "lact_newton_schulz", "lact_newton_schulz_static_capacity",
            "lact_newton_schulz_static", "lact_newton_schulz_backward_workspace_bytes", "lact_newton_schulz_backward",

@@ -161,6 +161,7 @@ static __device__ unsigned g_async_errors;
 namespace {
 bool g_overlap = true;
 bool g_fused_ns = true;
+int g_keep_pre = -1;       // LACT_OPT_KEEP_PREACTIVATIONS: -1 by shape, 0 never, 1 whenever the kernels allow it
 int g_persist = 1;          // hidden-stage kernels on the persistent engine (LACT_OPT_PERSISTENT_TILES): bit 0 apply, 1 update, 2 apply backward
                             // (the update's eight-output epilogue is faster staged through the whole ring by all eight waves: off by default)
 long long g_ns_spin_limit = NS_FUSED_SPIN_LIMIT;   // barrier wait bound of the fused Newton-Schulz kernels (lact_set_option)
@@ -365,7 +366,11 @@ struct Plan {
     const size_t sq3 = sq_total;
     s_ab = muon ? sv.take((size_t)nupd * std::max(1, S) * sq3 * nsz) : 0;
     s_bb = muon ? sv.take((size_t)nupd * std::max(1, S) * sq3 * nsz) : 0;
-    keep_pre = bf16 && d.d % 64 == 0 && d.dh % 64 == 0 && !d.forward_only;
+    // Keep the update's rounded pre-activations and lr-scaled operands for the backward (three GEMM phases there
+    // instead of six), or let the backward recompute them?  Recomputing costs K = d of matrix work per tile and saves
+    // five token-major arrays of stores in the forward: at d <= 128 (two K-steps) recomputing wins (d = 128, dh = 256,
+    // 32760 tokens: 3.61 against 3.70 ms per step), at d = 384 keeping does (1.298 against 1.316 ms; 7.38 against 7.47).
+    keep_pre = bf16 && d.d % 64 == 0 && d.dh % 64 == 0 && !d.forward_only && (g_keep_pre < 0 ? d.d > 128 : g_keep_pre != 0);
     s_pre.clear(); pre_T.clear();
     if (keep_pre)
       for (const auto& st : steps)
@@ -1877,6 +1882,11 @@ int lact_set_option(int32_t option, int32_t value) {
     const long long was = g_ns_spin_limit;
     g_ns_spin_limit = value > 0 ? value : NS_FUSED_SPIN_LIMIT;
     return (int)std::min<long long>(was, 0x7fffffff);
+  }
+  if (option == LACT_OPT_KEEP_PREACTIVATIONS) {
+    const int was = g_keep_pre;
+    g_keep_pre = value < 0 ? -1 : (value != 0);
+    return was;
   }
   if (option == LACT_OPT_PERSISTENT_TILES) {
     const int was = g_persist;

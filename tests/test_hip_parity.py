@@ -1129,9 +1129,9 @@ def test_stream_overlap_is_bit_identical(prenorm):
     (16, 2 * 1024 + 7, 384, 384, 1024, True),     # config-1 head shape, several tiles per block
     (1, 2 * 64, 64, 64, 64, False)])              # fewer tiles than compute units, one K-step per phase
 def test_persistent_tiles_are_bit_identical(b, L, d, dh, C, muon):
-    """The hidden-stage kernels as persistent blocks (copy waves running ahead across tiles and doing the previous
-    tile's epilogue beside the matrix waves) against one tile per block: the same arithmetic in the same order, so the
-    same bits in the output and in every gradient."""
+    """The hidden-stage kernels as persistent blocks (copy waves running ahead across tiles while the matrix waves run
+    the previous tile's epilogue) against one tile per block: the same arithmetic in the same order, so the same bits
+    in the output and in every gradient."""
     say("persistent tiles on/off", b, L, d, dh, C, muon)
     from lact_amd import _lib
     inp = problem(b, L, d, dh, seed=55, act=torch.bfloat16)
@@ -1159,6 +1159,42 @@ def test_persistent_tiles_are_bit_identical(b, L, d, dh, C, muon):
         for n in g0:
             assert torch.equal(g1[n], g0[n]), (n, O.rel_l2(g1[n], g0[n]))
     assert all(torch.equal(on[0][1][n], on[1][1][n]) for n in on[0][1])
+
+
+@pytest.mark.parametrize("b,L,d,dh,C,muon", [
+    (3, 3 * 256 + 40, 128, 256, 256, True),       # the shape class where the library recomputes by itself (d <= 128)
+    (2, 2 * 1024 + 7, 384, 384, 1024, True),      # ... and where it keeps
+    (2, 3 * 128, 64, 192, 128, False)])
+def test_kept_and_recomputed_update_backward_agree(b, L, d, dh, C, muon):
+    """The update's backward from the pre-activations the forward kept against the backward that recomputes them
+    (LACT_OPT_KEEP_PREACTIVATIONS 1 / 0): the recomputed products run over the same K-steps in the same order, so
+    the output and every gradient have the same bits -- except the learning-rate gradients, fp32 sums over a token's
+    hidden units that the two kernels take over tiles of different width (order of an fp32 sum: <= 1e-6)."""
+    say("keep / recompute", b, L, d, dh, C, muon)
+    from lact_amd import _lib
+    inp = problem(b, L, d, dh, seed=56, act=torch.bfloat16)
+    go = torch.randn(b, L, d, generator=torch.Generator().manual_seed(9)).bfloat16().to(DEV)
+
+    def run():
+        t = clone_to(inp, DEV)
+        out = T.block_causal_lact_swiglu(*args9(t), C, muon, t["momentum"])
+        g = grads_of(out, t, go)
+        torch.cuda.synchronize()
+        return out, g
+    L_ = _lib.lib()
+    prev = L_.lact_set_option(_lib.OPT_KEEP_PREACTIVATIONS, 1)
+    try:
+        o1, g1 = run()
+        L_.lact_set_option(_lib.OPT_KEEP_PREACTIVATIONS, 0)
+        o0, g0 = run()
+    finally:
+        L_.lact_set_option(_lib.OPT_KEEP_PREACTIVATIONS, prev)
+    assert torch.equal(o1, o0)
+    for n in g0:
+        if n in ("lr0", "lr1", "lr2"):
+            assert O.rel_l2(g1[n], g0[n]) <= 1e-6, (n, O.rel_l2(g1[n], g0[n]))
+        else:
+            assert torch.equal(g1[n], g0[n]), (n, O.rel_l2(g1[n], g0[n]))
 
 
 @pytest.mark.parametrize("chunks", [2, 3])
