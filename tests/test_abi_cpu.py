@@ -78,8 +78,10 @@ def test_query_sizes_and_validation_messages():
     assert "act_dtype" in err(make_desc(ops.block_causal_steps(256, 64), act_dtype=3))
     # a forward-only descriptor keeps less for the backward, and the backward entry point refuses it (before it
     # looks at any pointer: no GPU is needed for this check)
-    rc, saved_fo, _ = sizes(make_desc(ops.block_causal_steps(256, 64), forward_only=1))
-    assert rc == 0 and saved_fo < saved
+    # (at d = 256: the update's pre-activations are kept for the backward only above d = 128)
+    rc, saved_bw, _ = sizes(make_desc(ops.block_causal_steps(256, 64), d=256, dh=256))
+    rc_fo, saved_fo, _ = sizes(make_desc(ops.block_causal_steps(256, 64), d=256, dh=256, forward_only=1))
+    assert rc == 0 and rc_fo == 0 and saved_fo < saved_bw
     null = ctypes.c_void_p(0)
     fo = make_desc(ops.block_causal_steps(256, 64), forward_only=1)
     assert L.lact_backward(ctypes.byref(fo), *([null] * 22)) != 0
