@@ -200,8 +200,7 @@ class _LactProgramFn(torch.autograd.Function):
         res_out = out if out.dtype == out_dtype else out.to(out_dtype)
         if not prog.return_state:
             return (res_out, None, None, None, None, None, None)
-        m_ret = tuple(m if m is not None else torch.zeros_like(wf[i]) for i, m in enumerate(m_out))
-        return (res_out, w_out[0], w_out[1], w_out[2]) + m_ret
+        return (res_out, w_out[0], w_out[1], w_out[2]) + tuple(m_out)   # no momentum: no states (None), not zero tensors
 
     @staticmethod
     @torch.autograd.function.once_differentiable
@@ -247,7 +246,8 @@ class _LactProgramFn(torch.autograd.Function):
 
 @torch.compiler.disable
 def run_program(prog: Program, w0, w1, w2, q, k, v, lr0, lr1, lr2, momentum=None, momentum_state=None):
-    """Runs `prog`.  Returns (out, (w0, w1, w2) after the last update, (m0, m1, m2) momentum states).
+    """Runs `prog`.  Returns (out, (w0, w1, w2) after the last update, (m0, m1, m2) momentum states; None each
+    without momentum).
     `momentum_state` = the (m0, m1, m2) of an earlier call: the first update continues from it (inference only)."""
     res = _LactProgramFn.apply(prog, w0, w1, w2, q, k, v, lr0, lr1, lr2, momentum, momentum_state, torch.is_grad_enabled())
     return res[0], res[1:4], res[4:7]
