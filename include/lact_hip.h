@@ -209,7 +209,9 @@ int lact_set_option(int32_t option, int32_t value);
  * LACT_OPT_NS_BARRIER_SPIN_LIMIT) turns the step's results into NaN and adds one to a per-device counter that no
  * call clears.  lact_check_async_error copies that counter of the current device to the host (a synchronous copy: call
  * it once the stream the steps ran on has been synchronised), resets it and returns it: 0 = nothing happened, > 0 =
- * that many waits timed out since the last check (message in lact_last_error), < 0 = the check itself failed.  No
+ * that many waits timed out since the last check (message in lact_last_error; LACT_OPT_FUSED_NEWTON_SCHULZ is then
+ * switched off, so that the calls that follow cannot time out again, until the caller switches it back on), < 0 =
+ * the check itself failed.  No
  * counterpart in the reference, whose kernels never wait for each other.  The fused kernel is only used on a device
  * with at least 256 compute units (its groups must be resident as a whole); elsewhere the unfused launches run. */
 int lact_check_async_error(void);

@@ -2023,9 +2023,17 @@ int lact_check_async_error(void) {
   if (n == 0) return 0;
   const unsigned zero = 0;
   (void)hipMemcpyToSymbol(HIP_SYMBOL(g_async_errors), &zero, sizeof(zero), 0, hipMemcpyHostToDevice);
+  // Whatever held the compute units may still be there: later calls use the unfused launches, which wait for nobody,
+  // until the caller switches the fused kernel on again.
+  {
+    std::lock_guard<std::mutex> lock(g_enqueue_mutex);
+    g_fused_ns = false;
+  }
   g_err = std::to_string(n) + " barrier wait(s) of the fused Newton-Schulz kernel timed out on this device since the last check: "
-          "the results of those steps are NaN (compute units held by another process or kernel; raise "
-          "LACT_OPT_NS_BARRIER_SPIN_LIMIT or switch LACT_OPT_FUSED_NEWTON_SCHULZ off)";
+          "the results of those steps are NaN (compute units held by another process or kernel).  "
+          "LACT_OPT_FUSED_NEWTON_SCHULZ has been switched off: the calls that follow run three launches per iteration, "
+          "same results; switch it on again (and, if the waits are merely slow, raise LACT_OPT_NS_BARRIER_SPIN_LIMIT) "
+          "once the device is this process's alone";
   return (int)std::min<unsigned>(n, 0x7fffffffu);
 }
 

@@ -727,6 +727,9 @@ def test_fused_newton_schulz_barrier_timeout_ends_every_kernel_and_poisons_the_s
     with pytest.raises(RuntimeError, match="timed out"):
         ops.check_async_error()
     assert L.lact_check_async_error() == 0
+    # ... and the fused kernel is off from then on (whatever held the compute units may still be there): the caller
+    # switches it back on
+    assert L.lact_set_option(_lib.OPT_FUSED_NEWTON_SCHULZ, 1) == 0
     assert torch.equal(bad_out[:, :128], good_out[:, :128])      # first chunk: initial weights, no Newton-Schulz yet
     assert torch.isnan(bad_out[:, 128:]).all()                   # everything behind the first update
     assert torch.isnan(bad["w0"]).all() and torch.isnan(bad["k"][:, :128]).all()
