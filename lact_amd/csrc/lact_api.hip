@@ -695,7 +695,7 @@ struct Runner {
       HiddenDmaParams q;
       q.h = hp;
       (void)ver;
-      constexpr int SM3 = cmax(DmaSmem<TS_SQ, 2, 3>::BYTES, 4 * StageTile<TS_SQ, 2>::BYTES);   // k_update_hidden_dma stages four tiles at a time
+      constexpr int SM3 = DmaSmem<TS_SQ, 2, 3>::BYTES;   // the epilogues stage at most three bf16 tiles, inside the ring
       constexpr int SM6 = cmax(DmaSmem<TS_BWD, 2, 3>::BYTES, 6 * StageTile<TS_BWD, 2>::BYTES);
       const TileMap m3 = make_tile_map(ceil_div(T_, TS_SQ::BM), ceil_div(d.dh, TS_SQ::BN), d.b);
       const TileMap m6 = make_tile_map(ceil_div(T_, TS_BWD::BM), ceil_div(d.dh, TS_BWD::BN), d.b);
