@@ -372,6 +372,20 @@ __device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
 // kernel) then runs on all eight waves, row-wise -- a thread owns eight consecutive columns of four rows -- and every
 // output goes from registers straight to whole 16-byte row segments: half the vector-ALU time per thread and three
 // staged tiles instead of eight.  Element by element the same operations on the same rounded values as before.
+// The three accumulators of a hidden-stage tile, rounded to bf16, into three staged tiles at the start of the ring
+// (matrix waves only; the caller synchronises the block before anyone reads them).
+template <class TS>
+__device__ __forceinline__ void stage_three_products(char* smem, const f32x16 (&a02)[2][TS::TM][TS::TN], const f32x16 (&a1)[1][TS::TM][TS::TN]) {
+  using SB = StageTile<TS, 2>;
+  static_assert(3 * SB::BYTES <= DmaSmem<TS, 2, 3>::BYTES, "the three staged tiles lie in the ring");
+  char* s0 = smem + SB::lane_base(); char* s1 = s0 + SB::BYTES; char* s2 = s0 + 2 * SB::BYTES;
+  if (threadIdx.x < TS::THREADS) LACT_FOR_QUADS(TS) {
+    SB::put4(s0, tm, tn, g, a02[0][tm][tn][4 * g], a02[0][tm][tn][4 * g + 1], a02[0][tm][tn][4 * g + 2], a02[0][tm][tn][4 * g + 3]);
+    SB::put4(s1, tm, tn, g, a02[1][tm][tn][4 * g], a02[1][tm][tn][4 * g + 1], a02[1][tm][tn][4 * g + 2], a02[1][tm][tn][4 * g + 3]);
+    SB::put4(s2, tm, tn, g, a1[0][tm][tn][4 * g], a1[0][tm][tn][4 * g + 1], a1[0][tm][tn][4 * g + 2], a1[0][tm][tn][4 * g + 3]);
+  }
+}
+
 template <class TS>
 __global__ __launch_bounds__(DMA_THREADS) void k_update_hidden_dma(const HiddenDmaParams pp) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -380,16 +394,10 @@ __global__ __launch_bounds__(DMA_THREADS) void k_update_hidden_dma(const HiddenD
   if (!pp.map.locate(blockIdx.x, bx, by, z)) return;
   const int m0 = bx * TS::BM, n0 = by * TS::BN;
   using SB = StageTile<TS, 2>;
-  static_assert(3 * SB::BYTES <= DmaSmem<TS, 2, 3>::BYTES, "the three staged tiles lie in the ring");
   {
     f32x16 a02[2][TS::TM][TS::TN], a1[1][TS::TM][TS::TN];
     three_acc_mainloop<TS>(pp, smem, m0, n0, z, a02, a1);
-    char* s0 = smem + SB::lane_base(); char* s1 = s0 + SB::BYTES; char* s2 = s0 + 2 * SB::BYTES;
-    if (threadIdx.x < TS::THREADS) LACT_FOR_QUADS(TS) {
-      SB::put4(s0, tm, tn, g, a02[0][tm][tn][4 * g], a02[0][tm][tn][4 * g + 1], a02[0][tm][tn][4 * g + 2], a02[0][tm][tn][4 * g + 3]);
-      SB::put4(s1, tm, tn, g, a02[1][tm][tn][4 * g], a02[1][tm][tn][4 * g + 1], a02[1][tm][tn][4 * g + 2], a02[1][tm][tn][4 * g + 3]);
-      SB::put4(s2, tm, tn, g, a1[0][tm][tn][4 * g], a1[0][tm][tn][4 * g + 1], a1[0][tm][tn][4 * g + 2], a1[0][tm][tn][4 * g + 3]);
-    }
+    stage_three_products<TS>(smem, a02, a1);
   }
   __syncthreads();
   if (!SB::active()) return;
@@ -442,6 +450,9 @@ __global__ __launch_bounds__(DMA_THREADS) void k_update_hidden_dma(const HiddenD
   }
 }
 
+// apply backward, hidden stage: Y0 = X W0^T, Y2 = X W2^T, GH = dOut W1 -> O0 = silu(Y0) * Y2 (the hidden activation,
+// recomputed), O1 = d Y0, O2 = d Y2 (lact_swiglu_ffn.py:46-76).  Epilogue as in k_update_hidden_dma: three staged
+// products, the pointwise part on all eight waves, stores straight from registers.
 template <class TS>
 __global__ __launch_bounds__(DMA_THREADS) void k_apply_bwd_hidden_dma(const HiddenDmaParams pp) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -449,29 +460,46 @@ __global__ __launch_bounds__(DMA_THREADS) void k_apply_bwd_hidden_dma(const Hidd
   int bx, by, z;
   if (!pp.map.locate(blockIdx.x, bx, by, z)) return;
   const int m0 = bx * TS::BM, n0 = by * TS::BN;
-  f32x16 a02[2][TS::TM][TS::TN], a1[1][TS::TM][TS::TN];
-  three_acc_mainloop<TS>(pp, smem, m0, n0, z, a02, a1);
   using SB = StageTile<TS, 2>;
-  char* s0 = smem + SB::lane_base(); char* s1 = s0 + SB::BYTES; char* s2 = s0 + 2 * SB::BYTES;
-  if (threadIdx.x < TS::THREADS) LACT_FOR_QUADS(TS) {
-    float hq[4], gy0[4], gy2[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float y0 = round_bf16(a02[0][tm][tn][4 * g + j]), y2 = round_bf16(a02[1][tm][tn][4 * g + j]);
-      const float gh = round_bf16(a1[0][tm][tn][4 * g + j]);
-      const SiluParts s = silu_parts(y0);
-      const float sg = round_bf16(s.silu);
-      hq[j] = sg * y2; gy0[j] = round_bf16(gh * y2) * s.d1; gy2[j] = gh * sg;
-    }
-    SB::put4(s0, tm, tn, g, hq[0], hq[1], hq[2], hq[3]);
-    SB::put4(s1, tm, tn, g, gy0[0], gy0[1], gy0[2], gy0[3]);
-    SB::put4(s2, tm, tn, g, gy2[0], gy2[1], gy2[2], gy2[3]);
+  {
+    f32x16 a02[2][TS::TM][TS::TN], a1[1][TS::TM][TS::TN];
+    three_acc_mainloop<TS>(pp, smem, m0, n0, z, a02, a1);
+    stage_three_products<TS>(smem, a02, a1);
   }
   __syncthreads();
-  const size_t off = z * p.bso + (size_t)m0 * p.dh + n0;
-  copy_out_b16<TS>(smem + 0 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O0) + off, p.dh, p.T - m0, p.dh - n0);
-  copy_out_b16<TS>(smem + 1 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O1) + off, p.dh, p.T - m0, p.dh - n0);
-  copy_out_b16<TS>(smem + 2 * SB::BYTES, reinterpret_cast<uint16_t*>(p.O2) + off, p.dh, p.T - m0, p.dh - n0);
+  if (!SB::active()) return;
+  const int r0 = SB::row0(), c0 = SB::col0();
+  if (n0 + c0 >= p.dh) return;
+  const char* src = smem + (r0 * SB::LD + c0) * 2;
+  size_t off = z * p.bso + (size_t)(m0 + r0) * p.dh + n0 + c0;
+  const size_t step = (size_t)SB::RPP * p.dh;
+  uint4 u0[SB::PASSES], u2[SB::PASSES], ug[SB::PASSES];
+#pragma unroll
+  for (int ps = 0; ps < SB::PASSES; ++ps) {
+    u0[ps] = SB::read16(src, r0, ps);
+    u2[ps] = SB::read16(src + SB::BYTES, r0, ps);
+    ug[ps] = SB::read16(src + 2 * SB::BYTES, r0, ps);
+  }
+#pragma unroll
+  for (int ps = 0; ps < SB::PASSES; ++ps) {
+    const int r = r0 + ps * SB::RPP;
+    if (r < TS::BM && m0 + r < p.T) {
+      float y0[8], y2[8], gh[8], hq[8], gy0[8], gy2[8];
+      unpack8(u0[ps], y0);
+      unpack8(u2[ps], y2);
+      unpack8(ug[ps], gh);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const SiluParts sp = silu_parts(y0[j]);
+        const float sg = round_bf16(sp.silu);
+        hq[j] = sg * y2[j]; gy0[j] = round_bf16(gh[j] * y2[j]) * sp.d1; gy2[j] = gh[j] * sg;
+      }
+      *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(p.O0) + off) = pack8(hq);
+      *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(p.O1) + off) = pack8(gy0);
+      *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(p.O2) + off) = pack8(gy2);
+    }
+    off += step;
+  }
 }
 
 // update backward, hidden stage: phases (X; W0,W2), (X; G0,G2), (Y; W1T,G1T)
