@@ -647,88 +647,98 @@ __global__ __launch_bounds__(DMA_THREADS) void k_update_bwd_hidden_kept_dma(cons
     for (int i = 0; i < halves; ++i) __syncthreads();   // the input stages land behind these barriers
   }
   LACT_TS(2);
-  // input half h sits in the stage of K-step 2 nk + h
-  if (!loader) {
-    // the products enter the pointwise part as bf16 values: packing them in pairs first halves the registers
-    // the accumulators hold while that part runs
-    uint32_t pz[3][TS::TM][TS::TN][8];
+  // Input half h sits in the stage of K-step 2 nk + h; the stage of K-step 2 nk + 2 (= the last real K-step's, which
+  // every matrix wave has left: it has passed a barrier since its last fetch) is free.  Per half: the two matrix waves
+  // that own its 64 columns put their three rounded products there, in the layout of the input stage beside it; then
+  // all eight waves run the pointwise part row-wise -- a thread owns one 16-byte granule (8 columns) of two rows --
+  // and store the three results straight from registers.  Half the vector-ALU work per thread of a matrix-waves-only
+  // epilogue, and no staged result tiles.
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  char* fz = smem + ((2 * nk + 2) % STAGES) * SM::STAGE;
+  const size_t off = z * p.bso + (size_t)m0 * p.dh + n0;
+  for (int h = 0; h < halves; ++h) {
+    if (!loader && wave % TS::WAVES_N == h) {
+      const int row_l = (wave / TS::WAVES_N) * TS::WM + (lane & 31);
+      const uint32_t key = (uint32_t)((row_l >> 1) & 7) << 4;   // rows row_l + 32 tm share it
+      char* lb = fz + row_l * 128 + ((lane >> 5) << 3);
 #pragma unroll
-    for (int tm = 0; tm < TS::TM; ++tm)
+      for (int tm = 0; tm < TS::TM; ++tm)
 #pragma unroll
-      for (int tn = 0; tn < TS::TN; ++tn)
+        for (int tn = 0; tn < TS::TN; ++tn)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          pz[0][tm][tn][e] = (uint32_t)f32_to_bf16(ag[0][tm][tn][2 * e]) | ((uint32_t)f32_to_bf16(ag[0][tm][tn][2 * e + 1]) << 16);
-          pz[1][tm][tn][e] = (uint32_t)f32_to_bf16(ay[0][tm][tn][2 * e]) | ((uint32_t)f32_to_bf16(ay[0][tm][tn][2 * e + 1]) << 16);
-          pz[2][tm][tn][e] = (uint32_t)f32_to_bf16(ag[1][tm][tn][2 * e]) | ((uint32_t)f32_to_bf16(ag[1][tm][tn][2 * e + 1]) << 16);
-          // opaque to the optimiser: otherwise it undoes the packing and keeps every product as a float of its own
-          asm volatile("" : "+v"(pz[0][tm][tn][e]), "+v"(pz[1][tm][tn][e]), "+v"(pz[2][tm][tn][e]));
-        }
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int half = wave % TS::WAVES_N;
-    char* st = smem + ((2 * nk + half) % STAGES) * SM::STAGE;
-    const int row_l = (wave / TS::WAVES_N) * TS::WM + (lane & 31);
-    const uint32_t key = (uint32_t)((lane >> 1) & 7) << 4;
-    char* lb = st + row_l * 128 + ((lane >> 5) << 3);
+          for (int g = 0; g < 4; ++g) {
+            char* q0 = lb + tm * 32 * 128 + (((uint32_t)(tn * 4 + g) << 4) ^ key);
+            Elem<uint16_t>::store4(reinterpret_cast<uint16_t*>(q0), ag[0][tm][tn][4 * g], ag[0][tm][tn][4 * g + 1], ag[0][tm][tn][4 * g + 2], ag[0][tm][tn][4 * g + 3]);
+            Elem<uint16_t>::store4(reinterpret_cast<uint16_t*>(q0 + SM::A_BYTES), ay[0][tm][tn][4 * g], ay[0][tm][tn][4 * g + 1], ay[0][tm][tn][4 * g + 2], ay[0][tm][tn][4 * g + 3]);
+            Elem<uint16_t>::store4(reinterpret_cast<uint16_t*>(q0 + SM::A_BYTES + SM::B_BYTES), ag[1][tm][tn][4 * g], ag[1][tm][tn][4 * g + 1], ag[1][tm][tn][4 * g + 2], ag[1][tm][tn][4 * g + 3]);
+          }
+    }
+    __syncthreads();
+    const char* st = smem + ((2 * nk + h) % STAGES) * SM::STAGE;
+    const int j8 = threadIdx.x & 7;
+    uint4 ui[2][3], uz[2][3];
+    float l0[2], l1[2], l2[2];
 #pragma unroll
-    for (int tm = 0; tm < TS::TM; ++tm) {
-      const int ml = quad_m<TS>(tm), m = m0 + ml;
+    for (int ps = 0; ps < 2; ++ps) {
+      const int r = (threadIdx.x >> 3) + 64 * ps, m = m0 + r;
+      const uint32_t o = (uint32_t)(r * 128 + ((j8 ^ ((r >> 1) & 7)) << 4));
+      ui[ps][0] = *reinterpret_cast<const uint4*>(st + o);
+      ui[ps][1] = *reinterpret_cast<const uint4*>(st + SM::A_BYTES + o);
+      ui[ps][2] = *reinterpret_cast<const uint4*>(st + SM::A_BYTES + SM::B_BYTES + o);
+      uz[ps][0] = *reinterpret_cast<const uint4*>(fz + o);
+      uz[ps][1] = *reinterpret_cast<const uint4*>(fz + SM::A_BYTES + o);
+      uz[ps][2] = *reinterpret_cast<const uint4*>(fz + SM::A_BYTES + SM::B_BYTES + o);
       const bool mv = m < p.T;
-      const float l0 = mv ? p.lr0[z * p.bslr + m] : 0.f, l1 = mv ? p.lr1[z * p.bslr + m] : 0.f;
-      const float l2 = mv ? p.lr2[z * p.bslr + m] : 0.f;
+      l0[ps] = mv ? p.lr0[z * p.bslr + m] : 0.f;
+      l1[ps] = mv ? p.lr1[z * p.bslr + m] : 0.f;
+      l2[ps] = mv ? p.lr2[z * p.bslr + m] : 0.f;
+    }
+#pragma unroll
+    for (int ps = 0; ps < 2; ++ps) {
+      const int r = (threadIdx.x >> 3) + 64 * ps, m = m0 + r;
+      const bool mv = m < p.T;
+      float gg[8], h2[8], dh[8], gz0[8], gz1[8], gz2[8], o0[8], o1[8], o2[8];
+      unpack8(ui[ps][0], gg); unpack8(ui[ps][1], h2); unpack8(ui[ps][2], dh);
+      unpack8(uz[ps][0], gz0); unpack8(uz[ps][1], gz1); unpack8(uz[ps][2], gz2);
       float s0 = 0.f, s1 = 0.f, s2 = 0.f;
 #pragma unroll
-      for (int tn = 0; tn < TS::TN; ++tn)
+      for (int j = 0; j < 8; ++j) {
+        const SiluParts sp = silu_parts(gg[j]);
+        const UpdatePointwise u = update_pointwise<uint16_t>(gg[j], h2[j], dh[j], sp);
+        s0 += gz0[j] * u.dgpre; s1 += gz1[j] * u.hid; s2 += gz2[j] * u.dh2;
+        const float ghid = gz1[j] * l1[ps], gdh2 = gz2[j] * l2[ps], gdg = gz0[j] * l0[ps];
+        o0[j] = ghid * h2[j] * sp.d1 + gdh2 * dh[j] * sp.d1 + gdg * dh[j] * h2[j] * sp.d2;
+        o1[j] = gdh2 * sp.silu + gdg * h2[j] * sp.d1;
+        o2[j] = ghid * sp.silu + gdg * dh[j] * sp.d1;
+      }
+      // learning-rate gradients: the row's sum over this half's 64 columns (8 lanes), one partial per (row, half)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int nl = quad_n<TS>(tn, g);
-          const bool nv = n0 + nl < p.dh;
-          char* q0 = lb + tm * 32 * 128 + (((uint32_t)(tn * 4 + g) << 4) ^ key);
-          float i0[4], i1[4], i2[4], o0[4], o1[4], o2[4];
-          Elem<uint16_t>::load4(reinterpret_cast<const uint16_t*>(q0), i0);
-          Elem<uint16_t>::load4(reinterpret_cast<const uint16_t*>(q0 + SM::A_BYTES), i1);
-          Elem<uint16_t>::load4(reinterpret_cast<const uint16_t*>(q0 + SM::A_BYTES + SM::B_BYTES), i2);
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const float gg = i0[j], h2 = i1[j], dh = i2[j];
-            const uint32_t w0_ = pz[0][tm][tn][2 * g + (j >> 1)], w1_ = pz[1][tm][tn][2 * g + (j >> 1)], w2_ = pz[2][tm][tn][2 * g + (j >> 1)];
-            const float gz0 = __uint_as_float((j & 1) ? (w0_ & 0xffff0000u) : (w0_ << 16));
-            const float gz1 = __uint_as_float((j & 1) ? (w1_ & 0xffff0000u) : (w1_ << 16));
-            const float gz2 = __uint_as_float((j & 1) ? (w2_ & 0xffff0000u) : (w2_ << 16));
-            const SiluParts s = silu_parts(gg);
-            const UpdatePointwise u = update_pointwise<uint16_t>(gg, h2, dh, s);
-            if (mv && nv) { s0 += gz0 * u.dgpre; s1 += gz1 * u.hid; s2 += gz2 * u.dh2; }
-            const float ghid = gz1 * l1, gdh2 = gz2 * l2, gdg = gz0 * l0;
-            o0[j] = ghid * h2 * s.d1 + gdh2 * dh * s.d1 + gdg * dh * h2 * s.d2;
-            o1[j] = gdh2 * s.silu + gdg * h2 * s.d1;
-            o2[j] = ghid * s.silu + gdg * dh * s.d1;
-          }
-          Elem<uint16_t>::store4(reinterpret_cast<uint16_t*>(q0), o0[0], o0[1], o0[2], o0[3]);
-          Elem<uint16_t>::store4(reinterpret_cast<uint16_t*>(q0 + SM::A_BYTES), o1[0], o1[1], o1[2], o1[3]);
-          Elem<uint16_t>::store4(reinterpret_cast<uint16_t*>(q0 + SM::A_BYTES + SM::B_BYTES), o2[0], o2[1], o2[2], o2[3]);
+      for (int d = 1; d < 8; d <<= 1) {
+        s0 += __shfl_xor(s0, d, 64); s1 += __shfl_xor(s1, d, 64); s2 += __shfl_xor(s2, d, 64);
+      }
+      if (mv) {
+        const size_t o = off + (size_t)r * p.dh + h * 64 + j8 * 8;
+        *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(p.O0) + o) = pack8(o0);
+        *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(p.O1) + o) = pack8(o1);
+        *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(p.O2) + o) = pack8(o2);
+        if (j8 == 0) {
+          const size_t lo = (size_t)(by * TS::WAVES_N + h) * p.lrpart_stride + (size_t)z * p.Tcap + m;
+          p.lrpart[0 * p.lrpart_mat_stride + lo] = s0;
+          p.lrpart[1 * p.lrpart_mat_stride + lo] = s1;
+          p.lrpart[2 * p.lrpart_mat_stride + lo] = s2;
         }
-      store_row_partials<TS>(p, 0, tm, m, z, s0, by);
-      store_row_partials<TS>(p, 1, tm, m, z, s1, by);
-      store_row_partials<TS>(p, 2, tm, m, z, s2, by);
+      }
     }
+    if (h + 1 < halves) __syncthreads();   // the products of the next half go to the same place
   }
-  __syncthreads();
-  LACT_TS(3);
-  // copy the result stages out: 8 granules of 16 bytes per row and half, rows of 128 bytes stay whole
-  {
-    uint16_t* outs[3] = {reinterpret_cast<uint16_t*>(p.O0), reinterpret_cast<uint16_t*>(p.O1), reinterpret_cast<uint16_t*>(p.O2)};
-    const size_t off = z * p.bso + (size_t)m0 * p.dh + n0;
-    const int rows = min(TS::BM, p.T - m0);
-    for (int id = threadIdx.x; id < halves * TS::BM * 8; id += DMA_THREADS) {
-      const int j = id & 7, r = (id >> 3) % TS::BM, h = id / (8 * TS::BM);
-      if (r >= rows) continue;
-      const char* src = smem + ((2 * nk + h) % STAGES) * SM::STAGE + r * 128 + ((j ^ ((r >> 1) & 7)) << 4);
-      const size_t o = off + (size_t)r * p.dh + h * 64 + j * 8;
-      *reinterpret_cast<uint4*>(outs[0] + o) = *reinterpret_cast<const uint4*>(src);
-      *reinterpret_cast<uint4*>(outs[1] + o) = *reinterpret_cast<const uint4*>(src + SM::A_BYTES);
-      *reinterpret_cast<uint4*>(outs[2] + o) = *reinterpret_cast<const uint4*>(src + SM::A_BYTES + SM::B_BYTES);
+  // a half past the end of dh contributes nothing, but its slot of partial sums is read all the same
+  for (int h = halves; h < TS::WAVES_N; ++h)
+    if ((int)threadIdx.x < TS::BM && m0 + (int)threadIdx.x < p.T) {
+      const size_t lo = (size_t)(by * TS::WAVES_N + h) * p.lrpart_stride + (size_t)z * p.Tcap + m0 + threadIdx.x;
+      p.lrpart[0 * p.lrpart_mat_stride + lo] = 0.f;
+      p.lrpart[1 * p.lrpart_mat_stride + lo] = 0.f;
+      p.lrpart[2 * p.lrpart_mat_stride + lo] = 0.f;
     }
-  }
   LACT_TS(4);
 }
 
