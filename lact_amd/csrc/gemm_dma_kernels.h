@@ -538,56 +538,79 @@ __global__ __launch_bounds__(DMA_THREADS) void k_update_bwd_hidden_dma(const Hid
     pipe.template run_phase<2, false, true>(nk, step, ay);
   }
   __syncthreads();
+  // Epilogue: the six rounded products staged as bf16 tiles, then the pointwise part on all eight waves, row-wise (a
+  // thread owns 8 consecutive columns of two rows), results straight from registers to 16-byte row segments.
   using SB = StageTile<TS, 2>;
-  char* lb = smem + SB::lane_base();
-  if (!loader) {
-#pragma unroll
-  for (int tm = 0; tm < TS::TM; ++tm) {
-    const int ml = quad_m<TS>(tm), m = m0 + ml;
-    const bool mv = m < p.T;
-    const float l0 = mv ? p.lr0[z * p.bslr + m] : 0.f, l1 = mv ? p.lr1[z * p.bslr + m] : 0.f;
-    const float l2 = mv ? p.lr2[z * p.bslr + m] : 0.f;
-    float s0 = 0.f, s1 = 0.f, s2 = 0.f;
-#pragma unroll
-    for (int tn = 0; tn < TS::TN; ++tn)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int nl = quad_n<TS>(tn, g);
-        const bool nv = n0 + nl < p.dh;
-        float o0[4], o1[4], o2[4], o3[4], o4[4], o5[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float gg = round_bf16(aw[0][tm][tn][4 * g + j]), h2 = round_bf16(aw[1][tm][tn][4 * g + j]);
-          const float dh = round_bf16(ay[0][tm][tn][4 * g + j]);
-          const float gz0 = round_bf16(ag[0][tm][tn][4 * g + j]), gz2 = round_bf16(ag[1][tm][tn][4 * g + j]);
-          const float gz1 = round_bf16(ay[1][tm][tn][4 * g + j]);
-          const SiluParts s = silu_parts(gg);
-          const UpdatePointwise u = update_pointwise<uint16_t>(gg, h2, dh, s);
-          if (mv && nv) { s0 += gz0 * u.dgpre; s1 += gz1 * u.hid; s2 += gz2 * u.dh2; }
-          const float ghid = gz1 * l1, gdh2 = gz2 * l2, gdg = gz0 * l0;
-          o0[j] = ghid * h2 * s.d1 + gdh2 * dh * s.d1 + gdg * dh * h2 * s.d2;
-          o1[j] = gdh2 * s.silu + gdg * h2 * s.d1;
-          o2[j] = ghid * s.silu + gdg * dh * s.d1;
-          o3[j] = u.dgpre * l0; o4[j] = u.hid * l1; o5[j] = u.dh2 * l2;
-        }
-        SB::put4(lb + 0 * SB::BYTES, tm, tn, g, o0[0], o0[1], o0[2], o0[3]);
-        SB::put4(lb + 1 * SB::BYTES, tm, tn, g, o1[0], o1[1], o1[2], o1[3]);
-        SB::put4(lb + 2 * SB::BYTES, tm, tn, g, o2[0], o2[1], o2[2], o2[3]);
-        SB::put4(lb + 3 * SB::BYTES, tm, tn, g, o3[0], o3[1], o3[2], o3[3]);
-        SB::put4(lb + 4 * SB::BYTES, tm, tn, g, o4[0], o4[1], o4[2], o4[3]);
-        SB::put4(lb + 5 * SB::BYTES, tm, tn, g, o5[0], o5[1], o5[2], o5[3]);
-      }
-    store_row_partials<TS>(p, 0, tm, m, z, s0, by);
-    store_row_partials<TS>(p, 1, tm, m, z, s1, by);
-    store_row_partials<TS>(p, 2, tm, m, z, s2, by);
-  }
+  static_assert(TS::BN == 64 && TS::WAVES_N == 2, "a row is 8 granules: four per wave column");
+  {
+    char* lb = smem + SB::lane_base();
+    if (!loader) LACT_FOR_QUADS(TS) {
+      SB::put4(lb + 0 * SB::BYTES, tm, tn, g, aw[0][tm][tn][4 * g], aw[0][tm][tn][4 * g + 1], aw[0][tm][tn][4 * g + 2], aw[0][tm][tn][4 * g + 3]);
+      SB::put4(lb + 1 * SB::BYTES, tm, tn, g, aw[1][tm][tn][4 * g], aw[1][tm][tn][4 * g + 1], aw[1][tm][tn][4 * g + 2], aw[1][tm][tn][4 * g + 3]);
+      SB::put4(lb + 2 * SB::BYTES, tm, tn, g, ay[0][tm][tn][4 * g], ay[0][tm][tn][4 * g + 1], ay[0][tm][tn][4 * g + 2], ay[0][tm][tn][4 * g + 3]);
+      SB::put4(lb + 3 * SB::BYTES, tm, tn, g, ag[0][tm][tn][4 * g], ag[0][tm][tn][4 * g + 1], ag[0][tm][tn][4 * g + 2], ag[0][tm][tn][4 * g + 3]);
+      SB::put4(lb + 4 * SB::BYTES, tm, tn, g, ay[1][tm][tn][4 * g], ay[1][tm][tn][4 * g + 1], ay[1][tm][tn][4 * g + 2], ay[1][tm][tn][4 * g + 3]);
+      SB::put4(lb + 5 * SB::BYTES, tm, tn, g, ag[1][tm][tn][4 * g], ag[1][tm][tn][4 * g + 1], ag[1][tm][tn][4 * g + 2], ag[1][tm][tn][4 * g + 3]);
+    }
   }
   __syncthreads();
-  const size_t off = z * p.bso + (size_t)m0 * p.dh + n0;
-  void* outs[6] = {p.O0, p.O1, p.O2, p.O3, p.O4, p.O5};
+  const int r0 = SB::row0(), c0 = SB::col0();
+  const bool nv = n0 + c0 < p.dh;
+  const char* src = smem + (r0 * SB::LD + c0) * 2;
+  size_t off = z * p.bso + (size_t)(m0 + r0) * p.dh + n0 + c0;
+  const size_t step = (size_t)SB::RPP * p.dh;
+  uint4 u[SB::PASSES][6];
+  float l0[SB::PASSES], l1[SB::PASSES], l2[SB::PASSES];
 #pragma unroll
-  for (int i = 0; i < 6; ++i)
-    copy_out_b16<TS>(smem + i * SB::BYTES, reinterpret_cast<uint16_t*>(outs[i]) + off, p.dh, p.T - m0, p.dh - n0);
+  for (int ps = 0; ps < SB::PASSES; ++ps) {
+#pragma unroll
+    for (int i = 0; i < 6; ++i) u[ps][i] = SB::read16(src + i * SB::BYTES, r0, ps);
+    const int m = m0 + r0 + ps * SB::RPP;
+    const bool mv = r0 + ps * SB::RPP < TS::BM && m < p.T;
+    l0[ps] = mv ? p.lr0[z * p.bslr + m] : 0.f;
+    l1[ps] = mv ? p.lr1[z * p.bslr + m] : 0.f;
+    l2[ps] = mv ? p.lr2[z * p.bslr + m] : 0.f;
+  }
+#pragma unroll
+  for (int ps = 0; ps < SB::PASSES; ++ps) {
+    const int r = r0 + ps * SB::RPP, m = m0 + r;
+    const bool mv = r < TS::BM && m < p.T;
+    float gg[8], h2[8], dh[8], gz0[8], gz1[8], gz2[8], o0[8], o1[8], o2[8], o3[8], o4[8], o5[8];
+    unpack8(u[ps][0], gg); unpack8(u[ps][1], h2); unpack8(u[ps][2], dh);
+    unpack8(u[ps][3], gz0); unpack8(u[ps][4], gz1); unpack8(u[ps][5], gz2);
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const SiluParts sp = silu_parts(gg[j]);
+      const UpdatePointwise up = update_pointwise<uint16_t>(gg[j], h2[j], dh[j], sp);
+      if (mv && nv) { s0 += gz0[j] * up.dgpre; s1 += gz1[j] * up.hid; s2 += gz2[j] * up.dh2; }
+      const float ghid = gz1[j] * l1[ps], gdh2 = gz2[j] * l2[ps], gdg = gz0[j] * l0[ps];
+      o0[j] = ghid * h2[j] * sp.d1 + gdh2 * dh[j] * sp.d1 + gdg * dh[j] * h2[j] * sp.d2;
+      o1[j] = gdh2 * sp.silu + gdg * h2[j] * sp.d1;
+      o2[j] = ghid * sp.silu + gdg * dh[j] * sp.d1;
+      o3[j] = up.dgpre * l0[ps]; o4[j] = up.hid * l1[ps]; o5[j] = up.dh2 * l2[ps];
+    }
+    // learning-rate gradients: one partial per (row, wave column of 32 columns) = four lanes, slots as before
+    s0 += __shfl_xor(s0, 1, 64); s1 += __shfl_xor(s1, 1, 64); s2 += __shfl_xor(s2, 1, 64);
+    s0 += __shfl_xor(s0, 2, 64); s1 += __shfl_xor(s1, 2, 64); s2 += __shfl_xor(s2, 2, 64);
+    if (mv) {
+      if (nv) {
+        *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(p.O0) + off) = pack8(o0);
+        *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(p.O1) + off) = pack8(o1);
+        *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(p.O2) + off) = pack8(o2);
+        *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(p.O3) + off) = pack8(o3);
+        *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(p.O4) + off) = pack8(o4);
+        *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(p.O5) + off) = pack8(o5);
+      }
+      if ((threadIdx.x & 3) == 0) {
+        const size_t lo = (size_t)(by * TS::WAVES_N + ((threadIdx.x & 7) >> 2)) * p.lrpart_stride + (size_t)z * p.Tcap + m;
+        p.lrpart[0 * p.lrpart_mat_stride + lo] = s0;
+        p.lrpart[1 * p.lrpart_mat_stride + lo] = s1;
+        p.lrpart[2 * p.lrpart_mat_stride + lo] = s2;
+      }
+    }
+    off += step;
+  }
 }
 
 // update backward, hidden stage, from the pre-activations the forward kept (I0 = k W0^T, I1 = k W2^T, I2 = v W1,
