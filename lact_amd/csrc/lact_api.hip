@@ -446,7 +446,16 @@ void launch_row_gemm(const char* site, const RowGemmParams<NT>& p, int batch, hi
       RowGemmDmaParams<NT> q;
       q.g = p;
       q.out_ct = nullptr;
-      if (token_rows) launch_row_gemm_dma<TS_ROW, NT, EPI, !B_KC>(site, q, batch, s);
+      if (token_rows) {
+        // 256 x 128 tiles copy a third fewer operand bytes per FLOP than 128 x 128 ones, but a launch whose blocks fill
+        // the last round of compute units only partly wastes more than that: pick by the fuller last round
+        static const int cus = [] { int dev = 0, n = 0; (void)hipGetDevice(&dev); return hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0 ? n : 256; }();
+        auto fill = [&](int bm) { const long long blocks = (long long)ceil_div(p.M, bm) * ceil_div(p.N, 128) * batch; return (double)blocks / ((double)((blocks + cus - 1) / cus) * cus); };
+        // (measured at 384 blocks on 256 units: one-term GEMM 27.0 -> 24.5 us with the small tile, two-term GEMM with
+        // K-strided weights 34 -> 36 us: only the one-term case switches)
+        if (NT == 1 && fill(256) < 0.8 && fill(128) > fill(256) + 0.1) launch_row_gemm_dma<TS_SQ, NT, EPI, !B_KC>(site, q, batch, s);
+        else launch_row_gemm_dma<TS_ROW, NT, EPI, !B_KC>(site, q, batch, s);
+      }
       else if (p.M % TS_NS::BM == 0 && p.N % TS_NS::BN == 0) launch_row_gemm_dma<TS_NS, NT, EPI, !B_KC>(site, q, batch, s);
       else launch_row_gemm_dma<TS_SQ, NT, EPI, !B_KC>(site, q, batch, s);
       return;
