@@ -163,7 +163,8 @@ bool g_overlap = true;
 bool g_fused_ns = true;
 int g_keep_pre = -1;       // LACT_OPT_KEEP_PREACTIVATIONS: -1 by shape, 0 never, 1 whenever the kernels allow it
 int g_persist = 1;          // hidden-stage kernels on the persistent engine (LACT_OPT_PERSISTENT_TILES): bit 0 apply, 1 update, 2 apply backward
-                            // (the update's eight-output epilogue is faster staged through the whole ring by all eight waves: off by default)
+                            // (the one-tile-per-block kernels of the update and the apply backward, whose pointwise epilogues run on all
+                            // eight waves, measured faster than their persistent versions: only the apply's is on by default)
 long long g_ns_spin_limit = NS_FUSED_SPIN_LIMIT;   // barrier wait bound of the fused Newton-Schulz kernels (lact_set_option)
 std::mutex g_enqueue_mutex;   // one program is enqueued at a time (the side-stream context is shared)
 SideCtx* side_ctx() {
